@@ -1,0 +1,135 @@
+"""Pins the CPU oracle (oracle/bert_oracle.py) before anything trusts it."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from cudabert_amd import weights as W
+from cudabert_amd import synth
+from oracle import bert_oracle as O
+
+
+@pytest.fixture(scope="module")
+def tiny():
+    state = W.synth_state(W.TINY, seed=7, degenerate=False)
+    return W.to_npy_layout(state)
+
+
+@pytest.mark.parametrize("S", [5, 16, 33])
+def test_golden_tiny(tiny, golden_dir, S):
+    g = np.load(os.path.join(golden_dir, f"tiny_nd_s{S}.npz"))
+    seq, pooled, st = O.forward_torch(tiny, W.TINY.heads, g["ids"], g["seg"], g["mask"], return_stages=True)
+    assert np.abs(st["embedding"] - g["embedding"]).max() < 1e-5
+    assert np.abs(st["layer0"] - g["layer0"]).max() < 1e-5
+    assert np.abs(seq - g["seq"]).max() < 1e-5
+    assert np.abs(pooled - g["pooled"]).max() < 1e-5
+    seq64, pooled64 = O.forward_numpy64(tiny, W.TINY.heads, g["ids"], g["seg"], g["mask"])
+    assert np.abs(seq64 - g["seq"]).max() < 1e-5
+    assert np.abs(pooled64 - g["pooled"]).max() < 1e-5
+
+
+def test_golden_base_cfg0(golden_dir):
+    g = np.load(os.path.join(golden_dir, "base_cfg0_slice.npz"))
+    npy = W.to_npy_layout(W.synth_state(W.BASE, seed=20240, degenerate=True))
+    ids, seg, mask = synth.config_inputs(0)
+    assert (ids == g["ids"]).all() and (seg == g["seg"]).all() and (mask == g["mask"]).all()
+    seq, pooled = O.forward_torch(npy, W.BASE.heads, ids, seg, mask)
+    assert np.abs(pooled - g["pooled"]).max() < 1e-5
+    assert np.abs(seq[:, ::16, :32] - g["seq_slice"]).max() < 2e-5
+
+
+def test_torch_vs_numpy64_mask_none(tiny):
+    ids, seg, _ = synth.make_inputs(2, 9, [9, 9], vocab=W.TINY.vocab, seed=3)
+    a = O.forward_torch(tiny, 2, ids, seg, None)
+    b = O.forward_numpy64(tiny, 2, ids, seg, None)
+    c = O.forward_torch(tiny, 2, ids, seg, np.ones_like(ids))
+    for x, y, z in zip(a, b, c):
+        assert np.abs(x - y).max() < 1e-5
+        assert np.array_equal(x, z)          # all-ones mask == no mask
+
+
+def test_brute_force_attention_1x3():
+    """Head split / scale / mask / softmax / context written out with scalars
+    on B=1, S=3, A=2, d=2 -- a transposed operand or wrong head slicing fails."""
+    rng = np.random.default_rng(0)
+    B, S, A, d = 1, 3, 2, 2
+    H = A * d
+    x = rng.standard_normal((B, S, H)).astype(np.float32)
+    npy = {}
+    p = "bert_encoder_layer_0_"
+    for nm in ("query", "key", "value"):
+        npy[p + f"attention_self_{nm}_kernel"] = rng.standard_normal((H, H)).astype(np.float32)
+        npy[p + f"attention_self_{nm}_bias"] = rng.standard_normal(H).astype(np.float32)
+    mask = np.array([[1, 1, 0]])
+    got = O.self_attention_torch(torch.from_numpy(x), npy, p, A,
+                                 O.extended_mask_torch(torch.from_numpy(mask))).numpy()
+    q = x[0].astype(np.float64) @ npy[p + "attention_self_query_kernel"] + npy[p + "attention_self_query_bias"]
+    k = x[0].astype(np.float64) @ npy[p + "attention_self_key_kernel"] + npy[p + "attention_self_key_bias"]
+    v = x[0].astype(np.float64) @ npy[p + "attention_self_value_kernel"] + npy[p + "attention_self_value_bias"]
+    want = np.zeros((S, H))
+    for h in range(A):
+        for s in range(S):
+            sc = []
+            for t in range(S):
+                dot = sum(q[s, h * d + j] * k[t, h * d + j] for j in range(d))
+                sc.append(dot / math.sqrt(d) + (1 - mask[0, t]) * -10000.0)
+            m = max(sc)
+            e = [math.exp(z - m) for z in sc]
+            for j in range(d):
+                want[s, h * d + j] = sum(e[t] / sum(e) * v[t, h * d + j] for t in range(S))
+    assert np.abs(got[0] - want).max() < 1e-5
+
+
+def test_stage_closed_forms():
+    rng = np.random.default_rng(1)
+    x = torch.from_numpy(rng.standard_normal((7, 96)).astype(np.float32) * 3 + 1)
+    g = torch.from_numpy(rng.standard_normal(96).astype(np.float32))
+    b = torch.from_numpy(rng.standard_normal(96).astype(np.float32))
+    # LayerNorm against the library routine and against its moments.
+    ln = O.layer_norm_torch(x, g, b)
+    ref = torch.nn.functional.layer_norm(x, (96,), g, b, eps=1e-12)
+    assert (ln - ref).abs().max() < 1e-5
+    plain = O.layer_norm_torch(x, torch.ones(96), torch.zeros(96))
+    assert plain.mean(-1).abs().max() < 1e-5
+    assert (plain.var(-1, unbiased=False) - 1).abs().max() < 1e-4
+    # GELU: library erf form, known values, and NOT the tanh approximation.
+    ge = O.gelu_torch(x)
+    assert (ge - torch.nn.functional.gelu(x, approximate="none")).abs().max() < 1e-6
+    assert abs(O.gelu_torch(torch.tensor(1.0)).item() - 0.8413447460685429) < 1e-6
+    assert O.gelu_torch(torch.tensor(0.0)).item() == 0.0
+    # extended mask
+    m = O.extended_mask_torch(torch.tensor([[1, 0]]))
+    assert m.shape == (1, 1, 1, 2) and m.flatten().tolist() == [0.0, -10000.0]
+
+
+def test_invariants_padding_and_permutation(tiny):
+    ids, seg, mask = synth.make_inputs(3, 12, [12, 7, 3], vocab=W.TINY.vocab, seed=5)
+    seq, pooled = O.forward_torch(tiny, 2, ids, seg, mask)
+    # extra padding columns do not change outputs at valid positions
+    pad = lambda a: np.concatenate([a, np.zeros((3, 6), a.dtype)], axis=1)
+    seq2, pooled2 = O.forward_torch(tiny, 2, pad(ids), pad(seg), pad(mask))
+    for b, n in enumerate([12, 7, 3]):
+        assert np.abs(seq2[b, :n] - seq[b, :n]).max() < 1e-5
+    assert np.abs(pooled2 - pooled).max() < 1e-5
+    # permuting the batch permutes the outputs
+    perm = [2, 0, 1]
+    seq3, pooled3 = O.forward_torch(tiny, 2, ids[perm], seg[perm], mask[perm])
+    assert np.abs(seq3 - seq[perm]).max() < 1e-5
+    assert np.abs(pooled3 - pooled[perm]).max() < 1e-5
+    # pooled in (-1, 1): it is a tanh
+    assert np.abs(pooled).max() < 1.0
+
+
+def test_classifier_head(tiny):
+    rng = np.random.default_rng(2)
+    pooled = rng.standard_normal((4, W.TINY.hidden)).astype(np.float32)
+    p = O.classifier_head(tiny, pooled)
+    assert p.shape == (4, 2) and np.abs(p.sum(-1) - 1).max() < 1e-6
+    lin = torch.nn.Linear(W.TINY.hidden, 2)
+    lin.weight = torch.nn.Parameter(torch.tensor(tiny["classifier_kernel"].T))
+    lin.bias = torch.nn.Parameter(torch.tensor(tiny["classifier_bias"]))
+    with torch.no_grad():
+        ref = torch.softmax(lin(torch.from_numpy(pooled)), -1).numpy()
+    assert np.abs(p - ref).max() < 1e-6
