@@ -1,0 +1,201 @@
+// Fused self-attention for head dim 64 on gfx950:
+//   ctx = softmax(Q K^T * scale + maskadd) V        per (batch, head)
+//
+// One wave64 owns 32 query rows and walks the keys in blocks of 32 with an
+// online softmax, so the [S, S] score matrix never leaves registers.
+//
+// The score block is computed TRANSPOSED (keys x queries): K rows feed the
+// MFMA "A" operand and Q rows the "B" operand.  In the 32x32 accumulator
+// layout a lane then owns ONE query (column lane % 32) and 16 keys
+// (8*(v/4) + 4*(lane/32) + v%4), so the row maximum and row sum of the softmax
+// are 16 in-register operations plus one exchange with lane ^ 32.  The
+// probabilities stay in registers and feed the second MFMA as its "B" operand
+// (k = key); V is read from a pre-transposed [64, Sp] layout (written by the
+// QKV GEMM epilogue) so that the "A" operand lane (d, g) picks up the keys
+// that match the probability lane's k slots with 8/16-byte loads.  The
+// context comes out transposed too: a lane holds one query and four
+// consecutive head features per accumulator quad -> vector stores into the
+// row-major [tokens, hidden] context matrix.
+#include "kernels.h"
+
+namespace cubert {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <int ELT>
+__global__ __launch_bounds__(256) void attention_kernel(
+    const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
+    const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
+    unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale) {
+    constexpr int ES = (ELT == kBF16) ? 2 : 4;
+    constexpr int ROWB = 64 * ES;            // bytes per Q/K row
+    constexpr int KK = ROWB / 32;            // MFMA k-steps over the head dim (4 bf16 / 8 f32)
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, g = lane >> 5;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int q0 = (blockIdx.x * 4 + wave) * 32;
+    if (q0 >= S) return;                      // whole wave leaves; no barriers below
+
+    const size_t bh = (size_t)b * heads + h;
+    const unsigned char* qb = q + bh * S * ROWB;
+    const unsigned char* kb = k + bh * S * ROWB;
+    const unsigned char* vb = vt + bh * 64 * (size_t)Sp * ES;
+    const float* mrow = maskadd + (size_t)b * Sp;
+
+    // Q fragments ("B" operand: column = query), kept for the whole key loop.
+    int qrow = q0 + l32;
+    qrow = qrow < S ? qrow : S - 1;
+    uint4 qf[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+        qf[kk] = *reinterpret_cast<const uint4*>(qb + (size_t)qrow * ROWB + (2 * kk + g) * 16);
+
+    f32x16_t o[2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
+    float run_max = -INFINITY, run_sum = 0.0f;
+
+    for (int k0 = 0; k0 < S; k0 += 32) {
+        // ---- scores^T block: rows = keys k0..k0+31, column = my query ----
+        int krow = k0 + l32;
+        krow = krow < S ? krow : S - 1;
+        f32x16_t sc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const uint4 kf = *reinterpret_cast<const uint4*>(kb + (size_t)krow * ROWB + (2 * kk + g) * 16);
+            if constexpr (ELT == kBF16) {
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf),
+                                                             __builtin_bit_cast(bf16x8_t, qf[kk]), sc, 0, 0, 0);
+            } else {
+                const f32x4_t fa = __builtin_bit_cast(f32x4_t, kf);
+                const f32x4_t fb = __builtin_bit_cast(f32x4_t, qf[kk]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    sc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[e], fb[e], sc, 0, 0, 0);
+            }
+        }
+        // ---- scale + additive mask (padding columns carry -inf) ----
+        float blk_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f32x4_t m4 = *reinterpret_cast<const f32x4_t*>(mrow + k0 + 8 * j + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float s = sc[4 * j + e] * scale + m4[e];
+                sc[4 * j + e] = s;
+                blk_max = fmaxf(blk_max, s);
+            }
+        }
+        blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+        const float new_max = fmaxf(run_max, blk_max);    // finite: key 0 is never padding
+        const float alpha = __expf(run_max - new_max);    // exp(-inf) = 0 on the first block
+        float blk_sum = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float pv = __expf(sc[v] - new_max);
+            sc[v] = pv;
+            blk_sum += pv;
+        }
+        blk_sum += __shfl_xor(blk_sum, 32);
+        run_sum = run_sum * alpha + blk_sum;
+        run_max = new_max;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+
+        // ---- ctx^T += V^T (rows = head features) x P^T (column = my query) ----
+        if constexpr (ELT == kBF16) {
+#pragma unroll
+            for (int f = 0; f < 2; ++f) {        // keys k0 + 16 f + {4g..4g+3, 8+4g..8+4g+3}
+                bf16x8_t pf;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[e] = (__bf16)sc[8 * f + e];
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+                    const unsigned char* vrow = vb + ((size_t)(32 * db + l32) * Sp + k0 + 16 * f + 4 * g) * 2;
+                    const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                    const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                    const uint4 vf = {lo.x, lo.y, hi.x, hi.y};
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf), pf,
+                                                                  o[db], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {    // keys k0 + 8 j + 4 g + e
+                    const f32x4_t v4 = *reinterpret_cast<const f32x4_t*>(
+                        vb + ((size_t)(32 * db + l32) * Sp + k0 + 8 * j + 4 * g) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(v4[e], sc[4 * j + e], o[db], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- normalise and store: lane owns query q0 + l32, features 32 db + 8 j + 4 g + e ----
+    const int qi = q0 + l32;
+    if (qi >= S) return;
+    const float inv = 1.0f / run_sum;
+    const size_t hidden = (size_t)heads * 64;
+    unsigned char* orow = ctx + (((size_t)b * S + qi) * hidden + (size_t)h * 64) * ES;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = 32 * db + 8 * j + 4 * g;
+            if constexpr (ELT == kBF16) {
+                bf16x4_t w = {(__bf16)(o[db][4 * j] * inv), (__bf16)(o[db][4 * j + 1] * inv),
+                              (__bf16)(o[db][4 * j + 2] * inv), (__bf16)(o[db][4 * j + 3] * inv)};
+                *reinterpret_cast<bf16x4_t*>(orow + d * 2) = w;
+            } else {
+                f32x4_t w = {o[db][4 * j] * inv, o[db][4 * j + 1] * inv, o[db][4 * j + 2] * inv,
+                             o[db][4 * j + 3] * inv};
+                *reinterpret_cast<f32x4_t*>(orow + d * 4) = w;
+            }
+        }
+}
+
+}  // namespace
+
+bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
+                      int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream) {
+    if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
+    if (B <= 0 || heads <= 0 || S <= 0) { set_error("attention: empty problem"); return false; }
+    if (Sp % 32 != 0 || Sp < S || Sp - S >= 32) {
+        set_error("attention: Sp must be S rounded up to a multiple of 32");
+        return false;
+    }
+    if (B > 65535 || heads > 65535) { set_error("attention: grid too large"); return false; }
+    if (!q || !k || !vt || !maskadd || !ctx) { set_error("attention: null operand"); return false; }
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(vt) |
+         reinterpret_cast<uintptr_t>(maskadd) | reinterpret_cast<uintptr_t>(ctx)) & 15) {
+        set_error("attention: operands must be 16-byte aligned");
+        return false;
+    }
+    dim3 grid((S + 127) / 128, heads, B), block(256);
+    const unsigned char* qc = static_cast<const unsigned char*>(q);
+    const unsigned char* kc = static_cast<const unsigned char*>(k);
+    const unsigned char* vc = static_cast<const unsigned char*>(vt);
+    unsigned char* cc = static_cast<unsigned char*>(ctx);
+    if (elt == kBF16)
+        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale);
+    else
+        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale);
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+}  // namespace cubert

@@ -1,0 +1,274 @@
+// extern "C" surface of libcudaBERT.so (declared in include/cubert.h).
+#include "../../include/cubert.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "engine.h"
+#include "kernels.h"
+#include "weights.h"
+
+using cubert::Model;
+
+namespace {
+
+int env_int(const char* name, int dflt) {
+    const char* v = std::getenv(name);
+    if (!v || !*v) return dflt;
+    return std::atoi(v);
+}
+
+int env_precision() {
+    const char* v = std::getenv("CUBERT_PRECISION");
+    if (!v || !*v) return cubert::kF32;
+    const std::string s(v);
+    if (s == "bf16" || s == "BF16" || s == "1") return cubert::kBF16;
+    return cubert::kF32;
+}
+
+[[noreturn]] void die(const char* where) {
+    std::fprintf(stderr, "libcudaBERT: %s failed: %s\n", where, cubert::get_error());
+    std::fflush(stderr);
+    std::exit(EXIT_FAILURE);
+}
+
+Model* as_model(void* p, const char* where) {
+    if (!p) {
+        cubert::set_error(std::string(where) + ": model handle is NULL");
+        return nullptr;
+    }
+    return static_cast<Model*>(p);
+}
+
+void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const char* dir) {
+    cubert::ModelOptions opt;
+    opt.dims.hidden = cfg.hidden;
+    opt.dims.layers = cfg.layers;
+    opt.dims.heads = cfg.heads;
+    opt.dims.inter = cfg.intermediate;
+    opt.precision = cfg.precision;
+    opt.graph_max_tokens = cfg.graph_max_tokens;
+    opt.gpu = gpu;
+    opt.max_batch = maxB;
+    opt.max_seq = maxS;
+    opt.dir = dir ? dir : "";
+    return Model::create(opt);
+}
+
+cubert_config preset(bool large) {
+    // cuda_bert/utils/manager.cuh:46-50 (base) and manager.cu:8-15 (large)
+    cubert_config c;
+    c.hidden = large ? 1024 : 768;
+    c.layers = large ? 24 : 12;
+    c.heads = large ? 16 : 12;
+    c.intermediate = large ? 4096 : 3072;
+    c.precision = env_precision();
+    c.graph_max_tokens = env_int("CUBERT_GRAPH_MAX_TOKENS", 8192);
+    return c;
+}
+
+const char* default_dir(bool large) { return large ? "model_npy/large_uncased" : "model_npy/base_uncased"; }
+
+}  // namespace
+
+extern "C" {
+
+const char* cubert_last_error(void) { return cubert::get_error(); }
+
+void* init_model(bool large, int num_gpu, int max_batchsize, int max_seq_length, char* dir) {
+    cubert::set_error("");
+    const cubert_config c = preset(large);
+    const char* d = (dir && *dir) ? dir : default_dir(large);
+    return make_model(c, num_gpu, max_batchsize, max_seq_length, d);
+}
+
+void* init_model_ex(const cubert_config* cfg, int num_gpu, int max_batchsize, int max_seq_length, const char* dir) {
+    cubert::set_error("");
+    if (!cfg || !dir) { cubert::set_error("init_model_ex: cfg and dir must not be NULL"); return nullptr; }
+    return make_model(*cfg, num_gpu, max_batchsize, max_seq_length, dir);
+}
+
+void release_model(void* model) { delete static_cast<Model*>(model); }
+
+int cubert_check_weight_dir(const cubert_config* cfg, const char* dir) {
+    cubert::set_error("");
+    if (!cfg || !dir) { cubert::set_error("cubert_check_weight_dir: NULL argument"); return 1; }
+    cubert::Dims d;
+    d.hidden = cfg->hidden; d.layers = cfg->layers; d.heads = cfg->heads; d.inter = cfg->intermediate;
+    if (d.hidden != d.heads * 64) { cubert::set_error("head dimension must be 64 (hidden == 64 * heads)"); return 1; }
+    cubert::WeightDir wd;
+    return cubert::load_weight_dir(dir, &d, &wd) ? 0 : 1;
+}
+
+int cubert_encode(void* model, const int* words, const int* token_types, const int* attention_mask, int batchsize,
+                  int seq_length, float* pooled_out, float* seq_out, float* cls_out) {
+    cubert::set_error("");
+    Model* m = as_model(model, "cubert_encode");
+    if (!m) return 1;
+    if (!m->forward_host(words, token_types, attention_mask, batchsize, seq_length)) return 1;
+    if (cls_out && !m->classify()) return 1;
+    if (pooled_out && !m->copy_pooled(pooled_out)) return 1;
+    if (seq_out && !m->copy_seq(seq_out)) return 1;
+    if (cls_out && !m->copy_cls(cls_out)) return 1;
+    return m->sync() ? 0 : 1;
+}
+
+void Cuda_Bert(void* model, float* output, int* words, int* token_types, int batchsize, int seq_length,
+               int* attention_mask) {
+    if (!output) { cubert::set_error("output buffer is NULL"); die("Cuda_Bert"); }
+    if (cubert_encode(model, words, token_types, attention_mask, batchsize, seq_length, output, nullptr, nullptr) != 0)
+        die("Cuda_Bert");
+}
+
+Retval Cuda_Inference(void* model, int* words, int* token_types, int batchsize, int seq_length, int* masks) {
+    cubert::set_error("");
+    Model* m = as_model(model, "Cuda_Inference");
+    if (!m || !m->forward_host(words, token_types, masks, batchsize, seq_length)) die("Cuda_Inference");
+    Retval r;
+    r.tensor = m->seq_ptr();
+    r.pooled_output = m->pooled_ptr();
+    return r;
+}
+
+int cubert_forward_device(void* model, const int* d_words, const int* d_token_types, const int* d_attention_mask,
+                          int batchsize, int seq_length) {
+    cubert::set_error("");
+    Model* m = as_model(model, "cubert_forward_device");
+    if (!m) return 1;
+    return m->forward_device(d_words, d_token_types, d_attention_mask, batchsize, seq_length) ? 0 : 1;
+}
+
+int cubert_sync(void* model) {
+    Model* m = as_model(model, "cubert_sync");
+    return (m && m->sync()) ? 0 : 1;
+}
+
+float* cubert_seq_ptr(void* model) { return model ? static_cast<Model*>(model)->seq_ptr() : nullptr; }
+float* cubert_pooled_ptr(void* model) { return model ? static_cast<Model*>(model)->pooled_ptr() : nullptr; }
+void* cubert_stream(void* model) { return model ? static_cast<void*>(static_cast<Model*>(model)->stream()) : nullptr; }
+int cubert_hidden_size(void* model) { return model ? static_cast<Model*>(model)->dims().hidden : 0; }
+int cubert_num_classes(void* model) { return model ? static_cast<Model*>(model)->num_classes() : 0; }
+int cubert_precision(void* model) { return model ? static_cast<Model*>(model)->precision() : -1; }
+int cubert_graphs_cached(void* model) { return model ? static_cast<Model*>(model)->graphs_cached() : 0; }
+long cubert_capacity_tokens(void* model) { return model ? static_cast<Model*>(model)->capacity_tokens() : 0; }
+
+// Benchmark driver with the reference's inputs: the 11-token seed sentence is
+// repeated to the requested length with the last token kept at the end
+// (cuda_bert/cuda_bert.cu:12-22, 94-103).
+void test(int batchsize, int seq_length, int nIter, bool large, int num_gpu) {
+    static const int word_seed[11] = {2040, 2001, 3958, 27227, 1029, 3958, 103, 2001, 1037, 13997, 11510};
+    static const int type_seed[11] = {0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1};
+    static const int mask_seed[11] = {1, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0};
+    if (batchsize <= 0 || seq_length <= 0 || nIter <= 0) {
+        std::fprintf(stderr, "test: batchsize, seq_length and nIter must be positive\n");
+        return;
+    }
+    void* model = init_model(large, num_gpu, batchsize, seq_length, nullptr);
+    if (!model) die("test/init_model");
+    auto fill = [&](const int* seed) {
+        std::vector<int> row(seq_length);
+        for (int i = 0; i < seq_length - 1; ++i) row[i] = seed[i % 10];
+        row[seq_length - 1] = seed[10];
+        std::vector<int> all((size_t)batchsize * seq_length);
+        for (int b = 0; b < batchsize; ++b) std::memcpy(&all[(size_t)b * seq_length], row.data(), seq_length * sizeof(int));
+        return all;
+    };
+    std::vector<int> ids = fill(word_seed), seg = fill(type_seed), msk = fill(mask_seed);
+    const int hidden = cubert_hidden_size(model);
+    std::vector<float> out((size_t)batchsize * hidden);
+    std::printf(" Seq_length : %d\n Batchsize : %d\n%s\n", seq_length, batchsize,
+                large ? "Using large Model" : "Using Base Model");
+    for (int i = 0; i < 10; ++i) {
+        Cuda_Bert(model, out.data(), ids.data(), seg.data(), batchsize, seq_length, msk.data());
+        if (i == 0) {
+            std::printf("unit_test pooled[0][:10]:");
+            for (int j = 0; j < 10 && j < hidden; ++j) std::printf(" %.6f", out[j]);
+            std::printf("\n");
+        }
+    }
+    hipEvent_t start, stop;
+    hipStream_t stream = static_cast<hipStream_t>(cubert_stream(model));
+    if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) {
+        cubert::set_error("hipEventCreate failed");
+        die("test");
+    }
+    std::vector<float> latency(nIter);
+    double total = 0.0;
+    for (int i = 0; i < nIter; ++i) {
+        (void)hipEventRecord(start, stream);
+        Cuda_Bert(model, out.data(), ids.data(), seg.data(), batchsize, seq_length, msk.data());
+        (void)hipEventRecord(stop, stream);
+        (void)hipEventSynchronize(stop);
+        float ms = 0.0f;
+        (void)hipEventElapsedTime(&ms, start, stop);
+        latency[i] = ms;
+        total += ms;
+    }
+    std::sort(latency.begin(), latency.end());
+    std::printf(" 99 Latency : %fms\n", latency[std::min(nIter - 1, (int)(nIter * 0.99))]);
+    std::printf(" Throughput: %f lines per second\n", nIter * 1000.0 / total);
+    std::printf("Time= %.2f(ms)\n\n", total / nIter);
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+    release_model(model);
+}
+
+// ------------------------------------------------------------ single ops ---
+
+int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int M, int N, int K, int ldx, int elt,
+                   int out_elt, int epilogue, int tile, void* stream) {
+    cubert::set_error("");
+    if (epilogue < 0 || epilogue > 2) { cubert::set_error("cubert_op_gemm: epilogue must be 0, 1 or 2"); return 1; }
+    cubert::GemmParams p;
+    p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.elt = elt;
+    p.out_elt = out_elt; p.epilogue = epilogue; p.tile = tile;
+    return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q, void* k, void* vt, int B, int S,
+                       int heads, int elt, int tile, void* stream) {
+    cubert::set_error("");
+    if (B <= 0 || S <= 0 || heads <= 0) { cubert::set_error("cubert_op_gemm_qkv: bad shape"); return 1; }
+    cubert::GemmParams p;
+    p.X = X; p.W = W; p.bias = bias; p.M = B * S; p.N = 3 * heads * 64; p.K = heads * 64; p.ldx = heads * 64;
+    p.elt = elt; p.epilogue = cubert::kEpiQKV; p.q = q; p.k = k; p.vt = vt; p.S = S; p.Sp = cubert::round_up(S, 32);
+    p.heads = heads; p.tile = tile;
+    return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+int cubert_op_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx, int B,
+                        int heads, int S, float scale, int elt, void* stream) {
+    cubert::set_error("");
+    return cubert::launch_attention(q, k, vt, maskadd, ctx, B, heads, S, cubert::round_up(S > 0 ? S : 1, 32), scale,
+                                    elt, static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta, void* xb,
+                            int rows, int hidden, void* stream) {
+    cubert::set_error("");
+    return cubert::launch_add_layernorm(x, y, y_elt, gamma, beta, static_cast<cubert::bf16_t*>(xb), rows, hidden,
+                                        static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+int cubert_op_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word, const float* pos,
+                              const float* type, const float* gamma, const float* beta, float* x, void* xb,
+                              float* maskadd, int B, int S, int hidden, int vocab, int type_vocab, void* stream) {
+    cubert::set_error("");
+    return cubert::launch_embed_layernorm(ids, seg, mask, word, pos, type, gamma, beta, x,
+                                          static_cast<cubert::bf16_t*>(xb), maskadd, B, S,
+                                          cubert::round_up(S > 0 ? S : 1, 32), hidden, vocab, type_vocab,
+                                          static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+int cubert_op_mask_softmax(void* scores, int elt, const int* mask, int B, int rows_per_batch, int S, float scale,
+                           void* stream) {
+    cubert::set_error("");
+    return cubert::launch_mask_softmax(scores, elt, mask, B, rows_per_batch, S, scale,
+                                       static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+}  // extern "C"

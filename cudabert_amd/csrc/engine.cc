@@ -1,0 +1,354 @@
+#include "engine.h"
+
+#include <cmath>
+#include <cstring>
+
+#include "kernels.h"
+#include "weights.h"
+
+namespace cubert {
+
+namespace {
+
+thread_local std::string g_error;
+
+struct Arena {
+    size_t off = 0;
+    size_t take(size_t bytes) {
+        const size_t at = off;
+        off += (bytes + 255) / 256 * 256;
+        return at;
+    }
+};
+
+}  // namespace
+
+void set_error(const std::string& msg) { g_error = msg; }
+const char* get_error() { return g_error.c_str(); }
+
+Model* Model::create(const ModelOptions& opt) {
+    Model* m = new Model();
+    if (!m->init(opt)) {
+        const std::string keep = g_error;      // the destructor may issue HIP calls
+        delete m;
+        g_error = keep;
+        return nullptr;
+    }
+    return m;
+}
+
+Model::~Model() {
+    if (stream_) (void)hipStreamSynchronize(stream_);
+    for (auto& kv : graphs_)
+        if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+    if (wblock_) (void)hipFree(wblock_);
+    if (ablock_) (void)hipFree(ablock_);
+    if (h_in_) (void)hipHostFree(h_in_);
+    if (stream_) (void)hipStreamDestroy(stream_);
+}
+
+bool Model::init(const ModelOptions& opt_in) {
+    opt_ = opt_in;
+    Dims& D = opt_.dims;
+    if (opt_.precision != kF32 && opt_.precision != kBF16) { set_error("precision must be 0 (f32) or 1 (bf16)"); return false; }
+    if (D.hidden <= 0 || D.layers <= 0 || D.heads <= 0 || D.inter <= 0) { set_error("model dimensions must be positive"); return false; }
+    if (D.hidden != D.heads * 64) { set_error("head dimension must be 64 (hidden == 64 * heads)"); return false; }
+    if (D.hidden > 1024 || D.hidden % 64 != 0 || D.inter % 64 != 0) {
+        set_error("hidden must be a multiple of 64 up to 1024 and intermediate a multiple of 64");
+        return false;
+    }
+    if ((opt_.max_batch == 0) != (opt_.max_seq == 0) || opt_.max_batch < 0 || opt_.max_seq < 0) {
+        set_error("max_batchsize and max_seq_length must both be zero or both be positive");
+        return false;
+    }
+
+    // ---- host side first: nothing touches the GPU until the directory is valid ----
+    WeightDir wd;
+    if (!load_weight_dir(opt_.dir, &D, &wd)) return false;
+    if (opt_.max_seq > D.max_pos) {
+        set_error("max_seq_length " + std::to_string(opt_.max_seq) + " exceeds the position table (" +
+                  std::to_string(D.max_pos) + ")");
+        return false;
+    }
+    // Token capacity: explicit (B, S) as given, else the reference's default of
+    // 200*512 tokens (cuda_bert/utils/manager.cuh:55).
+    cap_tokens_ = opt_.max_batch ? (long)opt_.max_batch * opt_.max_seq : 200L * 512L;
+
+    int ndev = 0;
+    CUBERT_HIP_OK(hipGetDeviceCount(&ndev));
+    if (opt_.gpu < 0 || opt_.gpu >= ndev) {
+        set_error("GPU " + std::to_string(opt_.gpu) + " does not exist (" + std::to_string(ndev) + " visible)");
+        return false;
+    }
+    CUBERT_HIP_OK(hipSetDevice(opt_.gpu));
+    CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+
+    const int elt = opt_.precision;
+    const size_t es = elt == kBF16 ? 2 : 4;
+    const size_t H = D.hidden, I = D.inter;
+
+    // ---- weight block layout ----
+    Arena wa;
+    const size_t o_word = wa.take((size_t)D.vocab * H * 4), o_pos = wa.take((size_t)D.max_pos * H * 4),
+                 o_type = wa.take((size_t)D.type_vocab * H * 4), o_eg = wa.take(H * 4), o_eb = wa.take(H * 4);
+    struct LayerOff { size_t w_qkv, w_ao, w_in, w_out, b_qkv, b_ao, b_in, b_out, g1, be1, g2, be2; };
+    std::vector<LayerOff> lo(D.layers);
+    for (auto& l : lo) {
+        l.w_qkv = wa.take(3 * H * H * es); l.w_ao = wa.take(H * H * es);
+        l.w_in = wa.take(I * H * es); l.w_out = wa.take(H * I * es);
+        l.b_qkv = wa.take(3 * H * 4); l.b_ao = wa.take(H * 4); l.b_in = wa.take(I * 4); l.b_out = wa.take(H * 4);
+        l.g1 = wa.take(H * 4); l.be1 = wa.take(H * 4); l.g2 = wa.take(H * 4); l.be2 = wa.take(H * 4);
+    }
+    const size_t o_wp = wa.take(H * H * es), o_bp = wa.take(H * 4);
+    num_classes_ = wd.num_classes;
+    const size_t o_wc = wa.take((size_t)(num_classes_ ? num_classes_ : 1) * H * 4), o_bc = wa.take(8 * 4);
+    const size_t stage_floats = std::max(H * I, H * H);
+    const size_t o_stage = wa.take(stage_floats * 4);
+    weight_bytes_ = wa.off;
+    CUBERT_HIP_OK(hipMalloc(reinterpret_cast<void**>(&wblock_), weight_bytes_));
+
+    auto up = [&](size_t off, const NpyArray* a) -> bool {
+        CUBERT_HIP_OK(hipMemcpy(wblock_ + off, a->data.data(), a->data.size() * 4, hipMemcpyHostToDevice));
+        return true;
+    };
+    // [in, out] float32 on disk -> [out, in] operand type on device
+    float* stage = reinterpret_cast<float*>(wblock_ + o_stage);
+    auto up_t = [&](size_t off, const NpyArray* a) -> bool {
+        const int K = (int)a->shape[0], N = (int)a->shape[1];
+        CUBERT_HIP_OK(hipMemcpyAsync(stage, a->data.data(), a->data.size() * 4, hipMemcpyHostToDevice, stream_));
+        if (!launch_transpose_convert(stage, wblock_ + off, K, N, elt, stream_)) return false;
+        CUBERT_HIP_OK(hipStreamSynchronize(stream_));      // the staging buffer is reused
+        return true;
+    };
+    if (!up(o_word, wd.word) || !up(o_pos, wd.pos) || !up(o_type, wd.type) || !up(o_eg, wd.emb_g) || !up(o_eb, wd.emb_b))
+        return false;
+    word_ = reinterpret_cast<float*>(wblock_ + o_word);
+    pos_ = reinterpret_cast<float*>(wblock_ + o_pos);
+    type_ = reinterpret_cast<float*>(wblock_ + o_type);
+    emb_g_ = reinterpret_cast<float*>(wblock_ + o_eg);
+    emb_b_ = reinterpret_cast<float*>(wblock_ + o_eb);
+    layers_.resize(D.layers);
+    for (int i = 0; i < D.layers; ++i) {
+        const LayerTensors& T = wd.layers[i];
+        const LayerOff& l = lo[i];
+        // Q, K, V stacked along the output axis: rows [0,H) query, [H,2H) key, [2H,3H) value
+        // (the reference concatenates them too, cuda_bert/ops/linear.cu:60-88).
+        if (!up_t(l.w_qkv, T.q_k) || !up_t(l.w_qkv + H * H * es, T.k_k) || !up_t(l.w_qkv + 2 * H * H * es, T.v_k) ||
+            !up_t(l.w_ao, T.ao_k) || !up_t(l.w_in, T.in_k) || !up_t(l.w_out, T.out_k))
+            return false;
+        if (!up(l.b_qkv, T.q_b) || !up(l.b_qkv + H * 4, T.k_b) || !up(l.b_qkv + 2 * H * 4, T.v_b) ||
+            !up(l.b_ao, T.ao_b) || !up(l.b_in, T.in_b) || !up(l.b_out, T.out_b) || !up(l.g1, T.ao_g) ||
+            !up(l.be1, T.ao_be) || !up(l.g2, T.out_g) || !up(l.be2, T.out_be))
+            return false;
+        LayerDev& L = layers_[i];
+        L.w_qkv = wblock_ + l.w_qkv; L.w_ao = wblock_ + l.w_ao; L.w_in = wblock_ + l.w_in; L.w_out = wblock_ + l.w_out;
+        L.b_qkv = reinterpret_cast<float*>(wblock_ + l.b_qkv); L.b_ao = reinterpret_cast<float*>(wblock_ + l.b_ao);
+        L.b_in = reinterpret_cast<float*>(wblock_ + l.b_in); L.b_out = reinterpret_cast<float*>(wblock_ + l.b_out);
+        L.g1 = reinterpret_cast<float*>(wblock_ + l.g1); L.be1 = reinterpret_cast<float*>(wblock_ + l.be1);
+        L.g2 = reinterpret_cast<float*>(wblock_ + l.g2); L.be2 = reinterpret_cast<float*>(wblock_ + l.be2);
+    }
+    if (!up_t(o_wp, wd.pool_k) || !up(o_bp, wd.pool_b)) return false;
+    w_pool_ = wblock_ + o_wp;
+    b_pool_ = reinterpret_cast<float*>(wblock_ + o_bp);
+    if (num_classes_) {
+        if (!up(o_wc, wd.cls_k) || !up(o_bc, wd.cls_b)) return false;
+        w_cls_ = reinterpret_cast<float*>(wblock_ + o_wc);
+        b_cls_ = reinterpret_cast<float*>(wblock_ + o_bc);
+    }
+
+    // ---- activation block: one allocation, addresses fixed for the model's life ----
+    // B <= 1024 and every sequence is padded by < 32 key columns in vt/maskadd.
+    const size_t N = (size_t)cap_tokens_;
+    const size_t Npad = N + 32 * 1024;
+    Arena aa;
+    const size_t o_x32 = aa.take(N * H * 4);
+    const size_t o_xb = elt == kBF16 ? aa.take(N * H * 2) : 0;
+    const size_t o_q = aa.take((N + 64) * H * es), o_k = aa.take((N + 64) * H * es);
+    const size_t o_vt = aa.take(Npad * H * es), o_ctx = aa.take(N * H * es);
+    const size_t o_h = aa.take(N * I * es), o_y = aa.take(N * H * 4);
+    const size_t o_mask = aa.take(Npad * 4), o_pool = aa.take((size_t)1024 * H * 4), o_cls = aa.take(1024 * 8 * 4);
+    const size_t o_in = aa.take(3 * N * 4);
+    act_bytes_ = aa.off;
+    size_t free_b = 0, total_b = 0;
+    CUBERT_HIP_OK(hipMemGetInfo(&free_b, &total_b));
+    if (act_bytes_ > free_b) {
+        set_error("activation plan needs " + std::to_string(act_bytes_ >> 20) + " MiB but only " +
+                  std::to_string(free_b >> 20) + " MiB of device memory are free");
+        return false;
+    }
+    CUBERT_HIP_OK(hipMalloc(reinterpret_cast<void**>(&ablock_), act_bytes_));
+    // K rows past a sequence end and V^T padding columns are read (and then
+    // masked out); they must hold finite numbers, so start from all zeros.
+    CUBERT_HIP_OK(hipMemsetAsync(ablock_, 0, act_bytes_, stream_));
+    x32_ = reinterpret_cast<float*>(ablock_ + o_x32);
+    xb_ = elt == kBF16 ? reinterpret_cast<bf16_t*>(ablock_ + o_xb) : nullptr;
+    q_ = ablock_ + o_q; k_ = ablock_ + o_k; vt_ = ablock_ + o_vt; ctx_ = ablock_ + o_ctx; h_ = ablock_ + o_h;
+    y32_ = reinterpret_cast<float*>(ablock_ + o_y);
+    maskadd_ = reinterpret_cast<float*>(ablock_ + o_mask);
+    pooled_ = reinterpret_cast<float*>(ablock_ + o_pool);
+    cls_ = reinterpret_cast<float*>(ablock_ + o_cls);
+    d_in_ = reinterpret_cast<int*>(ablock_ + o_in);
+    CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_in_), 3 * N * 4, hipHostMallocDefault));
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    return true;
+}
+
+bool Model::check_shape(int B, int S) {
+    // Limits inherited from the reference: B*S within the allocated capacity
+    // (cuda_bert/utils/manager.cu:100-108), B <= 1024 (ops/batch_matmul.cu:60),
+    // S within the position table.
+    if (B <= 0 || S <= 0) { set_error("batchsize and seq_length must be positive"); return false; }
+    if (B > 1024) { set_error("batchsize " + std::to_string(B) + " exceeds 1024"); return false; }
+    if (S > opt_.dims.max_pos) {
+        set_error("seq_length " + std::to_string(S) + " exceeds the position table (" + std::to_string(opt_.dims.max_pos) + ")");
+        return false;
+    }
+    if ((long)B * S > cap_tokens_) {
+        set_error("batchsize * seq_length = " + std::to_string((long)B * S) + " exceeds the allocated capacity of " +
+                  std::to_string(cap_tokens_) + " tokens");
+        return false;
+    }
+    return true;
+}
+
+bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B, int S) {
+    if (!check_shape(B, S)) return false;
+    if (!ids || !seg) { set_error("input_ids and token_type_ids must not be null"); return false; }
+    const size_t n = (size_t)B * S, cap = (size_t)cap_tokens_;
+    const Dims& D = opt_.dims;
+    for (size_t i = 0; i < n; ++i) {
+        if ((unsigned)ids[i] >= (unsigned)D.vocab) {
+            set_error("input id " + std::to_string(ids[i]) + " at position " + std::to_string(i) + " is outside the vocabulary");
+            return false;
+        }
+        if ((unsigned)seg[i] >= (unsigned)D.type_vocab) {
+            set_error("token type " + std::to_string(seg[i]) + " at position " + std::to_string(i) + " is out of range");
+            return false;
+        }
+    }
+    // The pinned staging buffer is reused by every call: the previous upload
+    // must have left it before it is overwritten.
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    std::memcpy(h_in_, ids, n * 4);
+    std::memcpy(h_in_ + cap, seg, n * 4);
+    if (mask) std::memcpy(h_in_ + 2 * cap, mask, n * 4);
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_, h_in_, n * 4, hipMemcpyHostToDevice, stream_));
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + cap, h_in_ + cap, n * 4, hipMemcpyHostToDevice, stream_));
+    if (mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, h_in_ + 2 * cap, n * 4, hipMemcpyHostToDevice, stream_));
+    return run(B, S, mask != nullptr);
+}
+
+bool Model::forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S) {
+    if (!check_shape(B, S)) return false;
+    if (!d_ids || !d_seg) { set_error("input_ids and token_type_ids must not be null"); return false; }
+    const size_t n = (size_t)B * S, cap = (size_t)cap_tokens_;
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_, d_ids, n * 4, hipMemcpyDeviceToDevice, stream_));
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + cap, d_seg, n * 4, hipMemcpyDeviceToDevice, stream_));
+    if (d_mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, d_mask, n * 4, hipMemcpyDeviceToDevice, stream_));
+    return run(B, S, d_mask != nullptr);
+}
+
+bool Model::run(int B, int S, bool has_mask) {
+    B_ = B;
+    S_ = S;
+    const long tokens = (long)B * S;
+    if (opt_.graph_max_tokens <= 0 || tokens > opt_.graph_max_tokens) return enqueue(B, S, has_mask);
+    const long key = ((long)B * 1024 + S) * 2 + (has_mask ? 1 : 0);
+    GraphEntry& ge = graphs_[key];
+    if (ge.exec) {
+        CUBERT_HIP_OK(hipGraphLaunch(ge.exec, stream_));
+        return true;
+    }
+    if (ge.seen++ == 0) return enqueue(B, S, has_mask);      // first sight: run eagerly (one-time kernel setup)
+    // second sight: capture the launch sequence, then replay it
+    hipGraph_t graph = nullptr;
+    CUBERT_HIP_OK(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal));
+    const bool ok = enqueue(B, S, has_mask);
+    const std::string keep = ok ? std::string() : std::string(get_error());
+    const hipError_t e = hipStreamEndCapture(stream_, &graph);
+    if (!ok) { if (graph) (void)hipGraphDestroy(graph); set_error(keep); return false; }
+    if (e != hipSuccess) { set_error(std::string("hipStreamEndCapture failed: ") + hipGetErrorString(e)); return false; }
+    const hipError_t e2 = hipGraphInstantiate(&ge.exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e2 != hipSuccess) { ge.exec = nullptr; set_error(std::string("hipGraphInstantiate failed: ") + hipGetErrorString(e2)); return false; }
+    CUBERT_HIP_OK(hipGraphLaunch(ge.exec, stream_));
+    return true;
+}
+
+// The launch sequence of one forward pass (cuda_bert/utils/bert.cu:129-252):
+// 1 + 7 * layers + 1 kernels, no host synchronisation.
+bool Model::enqueue(int B, int S, bool has_mask) {
+    const Dims& D = opt_.dims;
+    const int elt = opt_.precision;
+    const int H = D.hidden, I = D.inter, N = B * S, Sp = round_up(S, 32);
+    const size_t cap = (size_t)cap_tokens_;
+    const int *ids = d_in_, *seg = d_in_ + cap, *mask = has_mask ? d_in_ + 2 * cap : nullptr;
+    const void* xin = elt == kBF16 ? static_cast<const void*>(xb_) : static_cast<const void*>(x32_);
+    const float scale = 1.0f / std::sqrt(64.0f);
+
+    if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32_, xb_, maskadd_, B, S, Sp, H,
+                                D.vocab, D.type_vocab, stream_))
+        return false;
+    for (int i = 0; i < D.layers; ++i) {
+        const LayerDev& L = layers_[i];
+        GemmParams g;
+        g.elt = elt;
+        // QKV projection, scattered per head (V transposed)
+        g.X = xin; g.ldx = H; g.W = L.w_qkv; g.bias = L.b_qkv; g.M = N; g.N = 3 * H; g.K = H;
+        g.epilogue = kEpiQKV; g.q = q_; g.k = k_; g.vt = vt_; g.S = S; g.Sp = Sp; g.heads = D.heads;
+        if (!launch_gemm(g, stream_)) return false;
+        if (!launch_attention(q_, k_, vt_, maskadd_, ctx_, B, D.heads, S, Sp, scale, elt, stream_)) return false;
+        // attention output projection -> f32, then residual add + LayerNorm
+        g = GemmParams();
+        g.elt = elt; g.out_elt = kF32; g.X = ctx_; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32_;
+        g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias;
+        if (!launch_gemm(g, stream_)) return false;
+        if (!launch_add_layernorm(x32_, y32_, kF32, L.g1, L.be1, xb_, N, H, stream_)) return false;
+        // feed-forward
+        g = GemmParams();
+        g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h_;
+        g.M = N; g.N = I; g.K = H; g.epilogue = kEpiBiasGelu;
+        if (!launch_gemm(g, stream_)) return false;
+        g = GemmParams();
+        g.elt = elt; g.out_elt = kF32; g.X = h_; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32_;
+        g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias;
+        if (!launch_gemm(g, stream_)) return false;
+        if (!launch_add_layernorm(x32_, y32_, kF32, L.g2, L.be2, xb_, N, H, stream_)) return false;
+    }
+    // pooler: tanh(dense(first token)); the first-token gather is the row stride S*H
+    GemmParams g;
+    g.elt = elt; g.out_elt = kF32; g.X = xin; g.ldx = S * H; g.W = w_pool_; g.bias = b_pool_; g.Y = pooled_;
+    g.M = B; g.N = H; g.K = H; g.epilogue = kEpiBiasTanh;
+    return launch_gemm(g, stream_);
+}
+
+bool Model::classify() {
+    if (!num_classes_) { set_error("the weight directory holds no classifier_kernel / classifier_bias"); return false; }
+    if (B_ <= 0) { set_error("classify() needs a preceding forward pass"); return false; }
+    return launch_classifier(pooled_, w_cls_, b_cls_, cls_, B_, opt_.dims.hidden, num_classes_, stream_);
+}
+
+bool Model::sync() {
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    return true;
+}
+
+bool Model::copy_pooled(float* out) {
+    if (!out || B_ <= 0) { set_error("no result to copy"); return false; }
+    CUBERT_HIP_OK(hipMemcpyAsync(out, pooled_, (size_t)B_ * opt_.dims.hidden * 4, hipMemcpyDeviceToHost, stream_));
+    return sync();
+}
+
+bool Model::copy_seq(float* out) {
+    if (!out || B_ <= 0) { set_error("no result to copy"); return false; }
+    CUBERT_HIP_OK(hipMemcpyAsync(out, x32_, (size_t)B_ * S_ * opt_.dims.hidden * 4, hipMemcpyDeviceToHost, stream_));
+    return sync();
+}
+
+bool Model::copy_cls(float* out) {
+    if (!out || B_ <= 0 || !num_classes_) { set_error("no result to copy"); return false; }
+    CUBERT_HIP_OK(hipMemcpyAsync(out, cls_, (size_t)B_ * num_classes_ * 4, hipMemcpyDeviceToHost, stream_));
+    return sync();
+}
+
+}  // namespace cubert

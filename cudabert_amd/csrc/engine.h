@@ -1,0 +1,101 @@
+// The encoder model: device-resident weights, a static activation plan and the
+// forward schedule.  Counterpart of `class bert` + `global_handle` of the
+// reference (cuda_bert/utils/bert.cu:4-252, utils/manager.cu:4-109).
+//
+// Differences that matter to callers: all device memory is allocated once at
+// construction (weights in one block, activations in one block sized for the
+// token capacity), every buffer address is a pure function of the model, there
+// are no host synchronisations inside the forward pass, and small batches are
+// replayed from a hipGraph captured per (batch, seq) shape.
+#pragma once
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace cubert {
+
+struct ModelOptions {
+    Dims dims;
+    int precision = kF32;      // operand type of the GEMMs and attention
+    int gpu = 0;
+    int max_batch = 0;         // (0, 0): default capacity of 200*512 tokens
+    int max_seq = 0;
+    int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
+    std::string dir;
+};
+
+struct LayerDev {
+    void *w_qkv, *w_ao, *w_in, *w_out;            // [out, in] in the operand type
+    float *b_qkv, *b_ao, *b_in, *b_out;
+    float *g1, *be1, *g2, *be2;
+};
+
+class Model {
+  public:
+    static Model* create(const ModelOptions& opt);     // nullptr + error text on failure
+    ~Model();
+
+    // Host inputs [B, S] int32 (mask may be nullptr).  Asynchronous.
+    bool forward_host(const int* ids, const int* seg, const int* mask, int B, int S);
+    // Inputs already in device memory.  Asynchronous on stream().
+    bool forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S);
+    // softmax(pooled @ classifier_kernel + bias) for the last forward -> cls_probs().
+    bool classify();
+    bool sync();
+    bool copy_pooled(float* host_out);                 // D2H + sync, B*hidden floats
+    bool copy_seq(float* host_out);                    // D2H + sync, B*S*hidden floats
+    bool copy_cls(float* host_out);                    // D2H + sync, B*num_classes floats
+
+    float* seq_ptr() const { return x32_; }
+    float* pooled_ptr() const { return pooled_; }
+    float* cls_ptr() const { return cls_; }
+    hipStream_t stream() const { return stream_; }
+    const Dims& dims() const { return opt_.dims; }
+    int precision() const { return opt_.precision; }
+    int num_classes() const { return num_classes_; }
+    long capacity_tokens() const { return cap_tokens_; }
+    int last_batch() const { return B_; }
+    int last_seq() const { return S_; }
+    int graphs_cached() const { return (int)graphs_.size(); }
+    size_t weight_bytes() const { return weight_bytes_; }
+    size_t activation_bytes() const { return act_bytes_; }
+
+  private:
+    Model() = default;
+    bool init(const ModelOptions& opt);
+    bool check_shape(int B, int S);
+    bool run(int B, int S, bool has_mask);             // graph or eager
+    bool enqueue(int B, int S, bool has_mask);         // the launch sequence
+
+    ModelOptions opt_;
+    hipStream_t stream_ = nullptr;
+    // weights
+    unsigned char* wblock_ = nullptr;
+    size_t weight_bytes_ = 0;
+    float *word_ = nullptr, *pos_ = nullptr, *type_ = nullptr, *emb_g_ = nullptr, *emb_b_ = nullptr;
+    std::vector<LayerDev> layers_;
+    void* w_pool_ = nullptr;
+    float* b_pool_ = nullptr;
+    float *w_cls_ = nullptr, *b_cls_ = nullptr;
+    int num_classes_ = 0;
+    // activations
+    unsigned char* ablock_ = nullptr;
+    size_t act_bytes_ = 0;
+    long cap_tokens_ = 0;
+    float* x32_ = nullptr;       // residual stream / sequence output [N, H] f32
+    bf16_t* xb_ = nullptr;       // bf16 copy of x (bf16 mode only)
+    void *q_ = nullptr, *k_ = nullptr, *vt_ = nullptr, *ctx_ = nullptr, *h_ = nullptr;
+    float* y32_ = nullptr;       // attn-out / ffn-out GEMM result [N, H] f32
+    float* maskadd_ = nullptr;   // [B, Sp]
+    float* pooled_ = nullptr;    // [B, H]
+    float* cls_ = nullptr;       // [B, C]
+    int* d_in_ = nullptr;        // ids | seg | mask, cap_tokens each
+    int* h_in_ = nullptr;        // pinned staging, same layout
+    int B_ = 0, S_ = 0;
+    struct GraphEntry { hipGraphExec_t exec = nullptr; int seen = 0; };
+    std::map<long, GraphEntry> graphs_;
+};
+
+}  // namespace cubert

@@ -1,0 +1,98 @@
+// Host-callable launchers for the gfx950 kernels.  Every launcher validates
+// the operand shapes its kernel and grid assume before launching and returns
+// false (with the error text set) instead of launching on a mismatch.
+//
+// Element types: `elt` selects the GEMM/attention operand type of a tensor --
+// 0 = float32, 1 = bfloat16 (stored as uint16).  Accumulation, LayerNorm and
+// softmax statistics are always float32.
+#pragma once
+#include "common.h"
+
+namespace cubert {
+
+// ---------------------------------------------------------------- GEMM -----
+// Y[m, n] = epilogue( sum_k X[m, k] * W[n, k] + bias[n] )
+//   X: [M, K] row-major with row stride ldx (elements), operand type `elt`
+//   W: [N, K] row-major (the on-disk [in,out] kernel transposed at load time)
+//   K must be a multiple of 128 bytes worth of elements (64 bf16 / 32 f32).
+// Replaces the cuBLAS calls + bias broadcast-fill of the reference
+// (cuda_bert/ops/linear.cu:91-148, 241-319; ops/matmul.cu:3-99).
+enum GemmEpilogue : int {
+    kEpiBias = 0,      // Y = acc + bias
+    kEpiBiasGelu = 1,  // Y = gelu_erf(acc + bias)       (ops/elementwise.cu:37-42 fused)
+    kEpiBiasTanh = 2,  // Y = tanh(acc + bias)           (ops/elementwise.cu:56-61 fused)
+    kEpiQKV = 3,       // scatter into per-head Q, K and transposed V (see below)
+};
+
+struct GemmParams {
+    const void* X = nullptr;
+    const void* W = nullptr;
+    const float* bias = nullptr;
+    void* Y = nullptr;        // [M, N] row-major, type out_elt (unused for kEpiQKV)
+    int M = 0, N = 0, K = 0;
+    int ldx = 0;              // row stride of X in elements (>= K)
+    int elt = kBF16;          // operand type of X and W
+    int out_elt = kBF16;      // type of Y
+    int epilogue = kEpiBias;
+    // kEpiQKV: N == 3*hidden.  Feature n -> (which = n / hidden, head, dd).
+    // Token m -> (b = m / S, s = m % S).  Outputs, all of operand type `elt`:
+    //   q  [B, heads, S, 64]      k  [B, heads, S, 64]     vt [B, heads, 64, Sp]
+    void* q = nullptr;
+    void* k = nullptr;
+    void* vt = nullptr;
+    int S = 0, Sp = 0, heads = 0;
+    int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile)
+};
+bool launch_gemm(const GemmParams& p, hipStream_t stream);
+
+// ----------------------------------------------------------- attention -----
+// Fused QK^T * scale + mask -> softmax -> P V for head dim 64.
+//   q, k [B, heads, S, 64], vt [B, heads, 64, Sp], maskadd [B, Sp] float
+//   (0 valid, -10000 masked, -inf for the padding columns S..Sp-1),
+//   ctx [B*S, heads*64] of type `elt`.
+// Replaces Query_Key / op_SoftMax / Prob_Value of the reference
+// (cuda_bert/ops/batch_matmul.cu:48-83,107-141; ops/softmax.cu:86-143)
+// without materialising the [B,S,heads,S] score tensor.
+bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd,
+                      void* ctx, int B, int heads, int S, int Sp, float scale, int elt,
+                      hipStream_t stream);
+
+// ----------------------------------------------------------- LayerNorm -----
+// x <- LayerNorm(x + y) * gamma + beta   over rows of length H, in place on the
+// float32 residual stream x; when xb != nullptr a bf16 copy of the result is
+// written as the next GEMM's operand.  y has type y_elt (may be nullptr: plain
+// LayerNorm).  eps = 1e-12 inside the square root, biased variance
+// (cuda_bert/ops/layernorm.cu:136-182; modeling.py:168-172).
+bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
+                          const float* beta, bf16_t* xb, int rows, int H, hipStream_t stream);
+
+// --------------------------------------------------- embedding + LN --------
+// x[t] = LayerNorm(word[ids[t]] + pos[t % S] + type[seg[t]]); also writes the
+// additive attention mask row maskadd[b, 0..Sp) (see launch_attention).  mask
+// may be nullptr (all positions valid).  ids/seg are clamped into range.
+// (cuda_bert/ops/embedding.cu:3-58; utils/bert.cu:94-97 for the positions.)
+bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
+                            const float* pos, const float* type, const float* gamma,
+                            const float* beta, float* x, bf16_t* xb, float* maskadd, int B, int S,
+                            int Sp, int H, int vocab, int type_vocab, hipStream_t stream);
+
+// ------------------------------------------------ scale+mask+softmax -------
+// In place over materialised scores [B, rows_per_batch, S] (float32 or bf16):
+// p = softmax(scores * scale + (1 - mask[b, :]) * -10000) along the last axis.
+// Stand-alone counterpart of cuApplySoftmax (cuda_bert/ops/softmax.cu:86-143).
+bool launch_mask_softmax(void* scores, int elt, const int* mask, int B, int rows_per_batch, int S,
+                         float scale, hipStream_t stream);
+
+// ------------------------------------------------------ classifier ---------
+// probs[b, :] = softmax(pooled[b, :] @ kernel[H, C] + bias[C]), C <= 8
+// (apps/finetune.py:16-24; the commented-out Cuda_Classify, cuda_bert.cu:72-89).
+bool launch_classifier(const float* pooled, const float* kernel, const float* bias, float* probs,
+                       int B, int H, int C, hipStream_t stream);
+
+// ------------------------------------------------------ load helpers -------
+// dst[n, k] = convert(src[k, n])  : on-disk [in,out] float32 -> [out,in] operand type.
+bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt,
+                              hipStream_t stream);
+bool launch_fill_f32(float* dst, float value, size_t n, hipStream_t stream);
+
+}  // namespace cubert

@@ -1,0 +1,345 @@
+// Bandwidth-bound row kernels for gfx950: residual-add + LayerNorm, embedding
+// gather + add + LayerNorm, scale + mask + softmax, classifier head and the
+// load-time weight transpose.  One wave64 owns one row; reductions are
+// butterfly shuffles over the 64 lanes, no LDS.
+#include "kernels.h"
+
+namespace cubert {
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+constexpr int kMaxChunks = 4;        // 4 chunks x 64 lanes x 4 elements = rows up to 1024
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// Normalises the row held in v[][] (lane owns elements c*256 + lane*4 + e) and
+// writes it to x (f32) and optionally xb (bf16).
+__device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H, int lane,
+                                                const float* __restrict__ gamma,
+                                                const float* __restrict__ beta, float* xrow,
+                                                bf16_t* xbrow) {
+    float s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if (c * 256 + lane * 4 < H) s += (v[c][0] + v[c][1]) + (v[c][2] + v[c][3]);
+    const float mean = wave_sum(s) / (float)H;
+    float sq = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        if (c * 256 + lane * 4 < H) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[c][e] -= mean;
+                sq += v[c][e] * v[c][e];
+            }
+        }
+    const float var = wave_sum(sq) / (float)H;
+    const float rstd = 1.0f / sqrtf(var + 1e-12f);
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+        const int i = c * 256 + lane * 4;
+        if (i < H) {
+            const f32x4_t g4 = *reinterpret_cast<const f32x4_t*>(gamma + i);
+            const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(beta + i);
+            f32x4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = g4[e] * (v[c][e] * rstd) + b4[e];
+            *reinterpret_cast<f32x4_t*>(xrow + i) = o;
+            if (xbrow) {
+                bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
+                *reinterpret_cast<bf16x4_t*>(xbrow + i) = ob;
+            }
+        }
+    }
+}
+
+template <int YELT>   // -1: no addend
+__global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ x,
+                                                            const unsigned char* __restrict__ y,
+                                                            const float* __restrict__ gamma,
+                                                            const float* __restrict__ beta,
+                                                            bf16_t* __restrict__ xb, int rows, int H) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    float* xrow = x + (size_t)row * H;
+    float v[kMaxChunks][4];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+        const int i = c * 256 + lane * 4;
+        if (i < H) {
+            f32x4_t a = *reinterpret_cast<const f32x4_t*>(xrow + i);
+            if constexpr (YELT == kF32) {
+                const f32x4_t t = *reinterpret_cast<const f32x4_t*>(y + ((size_t)row * H + i) * 4);
+                a += t;
+            } else if constexpr (YELT == kBF16) {
+                const bf16x4_t t = *reinterpret_cast<const bf16x4_t*>(y + ((size_t)row * H + i) * 2);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[e] += (float)t[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[c][e] = a[e];
+        }
+    }
+    normalise_store(v, H, lane, gamma, beta, xrow, xb ? xb + (size_t)row * H : nullptr);
+}
+
+__global__ __launch_bounds__(256) void embed_layernorm_kernel(
+    const int* __restrict__ ids, const int* __restrict__ seg, const int* __restrict__ mask,
+    const float* __restrict__ word, const float* __restrict__ pos, const float* __restrict__ type,
+    const float* __restrict__ gamma, const float* __restrict__ beta, float* __restrict__ x,
+    bf16_t* __restrict__ xb, float* __restrict__ maskadd, int B, int S, int Sp, int H, int vocab,
+    int type_vocab) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= B * S) return;
+    const int b = row / S, s = row - b * S;
+    int id = ids[row];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    int tt = seg ? seg[row] : 0;
+    tt = tt < 0 ? 0 : (tt >= type_vocab ? type_vocab - 1 : tt);
+    // additive attention mask: 0 valid, -10000 masked, -inf on the padding S..Sp-1
+    if (lane == 0) {
+        const int mk = mask ? mask[row] : 1;
+        maskadd[(size_t)b * Sp + s] = (1.0f - (float)mk) * -10000.0f;
+    }
+    if (s == 0 && S + lane < Sp) maskadd[(size_t)b * Sp + S + lane] = -INFINITY;   // Sp - S < 32
+    const float* wr = word + (size_t)id * H;
+    const float* pr = pos + (size_t)s * H;
+    const float* tr = type + (size_t)tt * H;
+    float v[kMaxChunks][4];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+        const int i = c * 256 + lane * 4;
+        if (i < H) {
+            const f32x4_t a = *reinterpret_cast<const f32x4_t*>(wr + i);
+            const f32x4_t p4 = *reinterpret_cast<const f32x4_t*>(pr + i);
+            const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(tr + i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[c][e] = (a[e] + p4[e]) + t4[e];
+        }
+    }
+    normalise_store(v, H, lane, gamma, beta, x + (size_t)row * H, xb ? xb + (size_t)row * H : nullptr);
+}
+
+// One wave per score row of length S <= 512 (8 elements per lane, strided by
+// 64 so that consecutive lanes touch consecutive elements).
+template <int ELT>
+__global__ __launch_bounds__(256) void mask_softmax_kernel(unsigned char* __restrict__ scores,
+                                                           const int* __restrict__ mask, long rows,
+                                                           int rows_per_batch, int S, float scale) {
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int b = (int)(row / rows_per_batch);
+    const int* mrow = mask ? mask + (size_t)b * S : nullptr;
+    unsigned char* base = scores + (size_t)row * S * (ELT == kBF16 ? 2 : 4);
+    float v[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int i = c * 64 + lane;
+        if (i < S) {
+            float s = (ELT == kBF16) ? (float)reinterpret_cast<const __bf16*>(base)[i]
+                                     : reinterpret_cast<const float*>(base)[i];
+            s = s * scale + (mrow ? (1.0f - (float)mrow[i]) * -10000.0f : 0.0f);
+            v[c] = s;
+            mx = fmaxf(mx, s);
+        }
+    }
+    mx = wave_max(mx);
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        if (c * 64 + lane < S) {
+            v[c] = expf(v[c] - mx);
+            sum += v[c];
+        }
+    const float inv = 1.0f / wave_sum(sum);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int i = c * 64 + lane;
+        if (i < S) {
+            if constexpr (ELT == kBF16) reinterpret_cast<__bf16*>(base)[i] = (__bf16)(v[c] * inv);
+            else reinterpret_cast<float*>(base)[i] = v[c] * inv;
+        }
+    }
+}
+
+// probs[b, :] = softmax(pooled[b, :] @ kernel[H, C] + bias); one wave per row.
+__global__ __launch_bounds__(64) void classifier_kernel(const float* __restrict__ pooled,
+                                                        const float* __restrict__ kernel,
+                                                        const float* __restrict__ bias,
+                                                        float* __restrict__ probs, int H, int C) {
+    const int lane = threadIdx.x, b = blockIdx.x;
+    float acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] = 0.0f;
+    for (int i = lane; i < H; i += 64) {
+        const float p = pooled[(size_t)b * H + i];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (c < C) acc[c] += p * kernel[(size_t)i * C + c];
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        if (c < C) {
+            acc[c] = wave_sum(acc[c]) + bias[c];
+            mx = fmaxf(mx, acc[c]);
+        }
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        if (c < C) {
+            acc[c] = expf(acc[c] - mx);
+            sum += acc[c];
+        }
+    if (lane == 0) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (c < C) probs[(size_t)b * C + c] = acc[c] / sum;
+    }
+}
+
+// dst[n, k] = src[k, n]; 32x32 tiles through LDS (padded against conflicts).
+template <int ELT>
+__global__ __launch_bounds__(256) void transpose_convert_kernel(const float* __restrict__ src,
+                                                                unsigned char* __restrict__ dst, int K,
+                                                                int N) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;      // 32 x 8
+    const int n0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const int kk = k0 + r, nn = n0 + tx;
+        tile[r][tx] = (kk < K && nn < N) ? src[(size_t)kk * N + nn] : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const int nn = n0 + r, kk = k0 + tx;
+        if (nn < N && kk < K) {
+            const float val = tile[tx][r];
+            if constexpr (ELT == kBF16) reinterpret_cast<__bf16*>(dst)[(size_t)nn * K + kk] = (__bf16)val;
+            else reinterpret_cast<float*>(dst)[(size_t)nn * K + kk] = val;
+        }
+    }
+}
+
+__global__ void fill_f32_kernel(float* dst, float value, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = value;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta,
+                          bf16_t* xb, int rows, int H, hipStream_t stream) {
+    if (rows <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
+        set_error("layernorm: H must be a multiple of 4 and at most 1024");
+        return false;
+    }
+    if (!x || !gamma || !beta || !aligned16(x) || !aligned16(gamma) || !aligned16(beta) ||
+        (y && !aligned16(y)) || (xb && !aligned16(xb))) {
+        set_error("layernorm: null or misaligned operand");
+        return false;
+    }
+    dim3 grid((rows + 3) / 4), block(256);
+    const unsigned char* yc = static_cast<const unsigned char*>(y);
+    if (!y) hipLaunchKernelGGL(add_layernorm_kernel<-1>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H);
+    else if (y_elt == kF32) hipLaunchKernelGGL(add_layernorm_kernel<kF32>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H);
+    else if (y_elt == kBF16) hipLaunchKernelGGL(add_layernorm_kernel<kBF16>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H);
+    else { set_error("layernorm: bad addend type"); return false; }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
+                            const float* pos, const float* type, const float* gamma, const float* beta,
+                            float* x, bf16_t* xb, float* maskadd, int B, int S, int Sp, int H, int vocab,
+                            int type_vocab, hipStream_t stream) {
+    if (B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
+        set_error("embedding: H must be a multiple of 4 and at most 1024");
+        return false;
+    }
+    if (Sp < S || Sp - S >= 32 || Sp % 32 != 0) { set_error("embedding: bad padded length"); return false; }
+    if (!ids || !word || !pos || !type || !gamma || !beta || !x || !maskadd || vocab <= 0 || type_vocab <= 0) {
+        set_error("embedding: null operand");
+        return false;
+    }
+    if (!aligned16(word) || !aligned16(pos) || !aligned16(type) || !aligned16(gamma) || !aligned16(beta) ||
+        !aligned16(x) || (xb && !aligned16(xb))) {
+        set_error("embedding: misaligned operand");
+        return false;
+    }
+    const long rows = (long)B * S;
+    dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    hipLaunchKernelGGL(embed_layernorm_kernel, grid, block, 0, stream, ids, seg, mask, word, pos, type, gamma,
+                       beta, x, xb, maskadd, B, S, Sp, H, vocab, type_vocab);
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_mask_softmax(void* scores, int elt, const int* mask, int B, int rows_per_batch, int S, float scale,
+                         hipStream_t stream) {
+    if (B <= 0 || rows_per_batch <= 0 || S <= 0 || S > 512) {
+        set_error("softmax: row length must be in 1..512");
+        return false;
+    }
+    if (!scores) { set_error("softmax: null operand"); return false; }
+    const long rows = (long)B * rows_per_batch;
+    const long blocks = (rows + 3) / 4;
+    if (blocks > 0x7fffffffL) { set_error("softmax: too many rows"); return false; }
+    dim3 grid((unsigned)blocks), block(256);
+    unsigned char* sc = static_cast<unsigned char*>(scores);
+    if (elt == kBF16) hipLaunchKernelGGL(mask_softmax_kernel<kBF16>, grid, block, 0, stream, sc, mask, rows, rows_per_batch, S, scale);
+    else if (elt == kF32) hipLaunchKernelGGL(mask_softmax_kernel<kF32>, grid, block, 0, stream, sc, mask, rows, rows_per_batch, S, scale);
+    else { set_error("softmax: bad element type"); return false; }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_classifier(const float* pooled, const float* kernel, const float* bias, float* probs, int B, int H,
+                       int C, hipStream_t stream) {
+    if (B <= 0 || H <= 0 || C <= 0 || C > 8) { set_error("classifier: supports 1..8 classes"); return false; }
+    if (!pooled || !kernel || !bias || !probs) { set_error("classifier: null operand"); return false; }
+    hipLaunchKernelGGL(classifier_kernel, dim3(B), dim3(64), 0, stream, pooled, kernel, bias, probs, H, C);
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt, hipStream_t stream) {
+    if (!src || !dst || K <= 0 || N <= 0) { set_error("transpose: bad arguments"); return false; }
+    dim3 grid((N + 31) / 32, (K + 31) / 32), block(256);
+    unsigned char* d = static_cast<unsigned char*>(dst);
+    if (elt == kBF16) hipLaunchKernelGGL(transpose_convert_kernel<kBF16>, grid, block, 0, stream, src, d, K, N);
+    else if (elt == kF32) hipLaunchKernelGGL(transpose_convert_kernel<kF32>, grid, block, 0, stream, src, d, K, N);
+    else { set_error("transpose: bad element type"); return false; }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_fill_f32(float* dst, float value, size_t n, hipStream_t stream) {
+    if (!dst || n == 0) return true;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, dst, value, n);
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+}  // namespace cubert

@@ -1,0 +1,159 @@
+/* C ABI of libcudaBERT.so, the MI355X (gfx950) BERT encoder inference engine.
+ *
+ * The first five entry points are exactly what the reference's ctypes binding
+ * loads (cuda_bert/pybert.py:12-38) and what cuda_model.py's Cuda_BERT calls;
+ * they keep the reference's names, argument order and meaning
+ * (cuda_bert/cuda_bert.cu:24-181).  Everything after them is additive.
+ *
+ * All `int*` inputs are C-contiguous int32 [batchsize, seq_length].  A model
+ * handle is not thread-safe (as in the reference); use one per host thread.
+ */
+#ifndef CUBERT_H_
+#define CUBERT_H_
+
+#include <stdbool.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------
+ * Reference-compatible entry points
+ * ---------------------------------------------------------------------- */
+
+/* Device pointers returned by Cuda_Inference (cuda_bert/utils/common.h:173-177):
+ * tensor = sequence output [B, S, hidden] float32, pooled_output = [B, hidden]
+ * float32.  Valid until the next call on the same model. */
+typedef struct Retval {
+    float* tensor;
+    float* pooled_output;
+} Retval;
+
+/* Replaces init_model (cuda_bert/cuda_bert.cu:26-33).  `large` selects
+ * BERT-large (24 x 1024 x 16 heads x 4096) or BERT-base (12 x 768 x 12 x 3072)
+ * as in cuda_bert/utils/manager.cu:8-15; `num_gpu` is the device ordinal;
+ * (max_batchsize, max_seq_length) size the activation memory, (0, 0) gives the
+ * reference's default capacity of 200*512 tokens; `dir` is the .npy weight
+ * directory ("" -> model_npy/base_uncased or model_npy/large_uncased).
+ * Precision and graph use come from the environment: CUBERT_PRECISION=fp32
+ * (default) | bf16, CUBERT_GRAPH_MAX_TOKENS (default 8192, 0 disables graphs).
+ * Returns NULL on failure (the reference exits the process); the reason is
+ * available from cubert_last_error(). */
+void* init_model(bool large, int num_gpu, int max_batchsize, int max_seq_length, char* dir);
+
+/* Replaces release_model (cuda_bert/cuda_bert.cu:34-37). */
+void release_model(void* model);
+
+/* Replaces Cuda_Bert (cuda_bert/cuda_bert.cu:55-70): runs the encoder on host
+ * inputs and writes batchsize*hidden float32 pooled outputs to the host buffer
+ * `output`; synchronous.  attention_mask may be NULL (no masking).  On an
+ * invalid call (shape over capacity, id out of range, device failure) it
+ * prints the reason to stderr and terminates the process with
+ * exit(EXIT_FAILURE), which is what the reference does through its asserts
+ * and checkCudaErrors (cuda_bert/utils/manager.cu:100-108, common.h:58-65).
+ * Callers that want an error code use cubert_encode instead. */
+void Cuda_Bert(void* model, float* output, int* words, int* token_types, int batchsize,
+               int seq_length, int* attention_mask);
+
+/* Replaces Cuda_Inference (cuda_bert/cuda_bert.cu:40-53): same forward pass,
+ * asynchronous, returns device pointers.  Call cubert_sync (or any later
+ * synchronous entry point) before reading them from another stream. */
+Retval Cuda_Inference(void* model, int* words, int* token_types, int batchsize, int seq_length,
+                      int* masks);
+
+/* Replaces test (cuda_bert/cuda_bert.cu:91-180; cuda_bert.cuh:4-5): loads the
+ * default weight directory, tiles the reference's 11-token seed input to
+ * (batchsize, seq_length), runs 10 warm-up and nIter timed iterations of
+ * forward + pooled-output copy and prints the 99th-percentile latency and the
+ * throughput in batches per second. */
+void test(int batchsize, int seq_length, int nIter, bool large, int num_gpu);
+
+/* ------------------------------------------------------------------------
+ * Additive entry points (no counterpart in the reference unless noted)
+ * ---------------------------------------------------------------------- */
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* cubert_last_error(void);
+
+typedef struct cubert_config {
+    int hidden, layers, heads, intermediate; /* head dim (hidden/heads) must be 64 */
+    int precision;                           /* 0 = float32, 1 = bfloat16 operands / float32 accumulate */
+    int graph_max_tokens;                    /* hipGraph replay for batches up to this many tokens; 0 = off */
+} cubert_config;
+
+/* init_model with explicit dimensions and precision. */
+void* init_model_ex(const cubert_config* cfg, int num_gpu, int max_batchsize, int max_seq_length,
+                    const char* dir);
+
+/* Host-only validation of a weight directory against cfg (names, dtypes,
+ * shapes); touches no GPU.  Returns 0 if init_model_ex would accept it. */
+int cubert_check_weight_dir(const cubert_config* cfg, const char* dir);
+
+/* Cuda_Bert with an error code instead of process exit.  Any of pooled_out
+ * [B, hidden], seq_out [B, S, hidden] and cls_out [B, num_classes] may be NULL.
+ * cls_out is the fine-tune head softmax(pooled @ classifier_kernel + bias) --
+ * the reference's commented-out Cuda_Classify (cuda_bert/cuda_bert.cu:72-89)
+ * and apps/finetune.py:16-44 run on the device.  Returns 0 on success. */
+int cubert_encode(void* model, const int* words, const int* token_types, const int* attention_mask,
+                  int batchsize, int seq_length, float* pooled_out, float* seq_out, float* cls_out);
+
+/* Forward pass on inputs that already live in device memory; asynchronous on
+ * the model's stream.  Returns 0 on success. */
+int cubert_forward_device(void* model, const int* d_words, const int* d_token_types,
+                          const int* d_attention_mask, int batchsize, int seq_length);
+int cubert_sync(void* model);
+
+/* Introspection. */
+float* cubert_seq_ptr(void* model);       /* device, [B, S, hidden] float32 */
+float* cubert_pooled_ptr(void* model);    /* device, [B, hidden] float32 */
+void* cubert_stream(void* model);         /* hipStream_t the model enqueues on */
+int cubert_hidden_size(void* model);
+int cubert_num_classes(void* model);
+int cubert_precision(void* model);
+int cubert_graphs_cached(void* model);
+long cubert_capacity_tokens(void* model);
+
+/* ---- single kernels on caller-owned device memory (parity tests, roofline
+ * timing).  `stream` is a hipStream_t (NULL = default stream); elt: 0 float32,
+ * 1 bfloat16.  All return 0 on success. ---- */
+
+/* Y[M,N] = epilogue(X[M,K] (row stride ldx) * W[N,K]^T + bias[N]);
+ * epilogue 0 bias, 1 bias+GELU(erf), 2 bias+tanh.  tile 0 = automatic.
+ * Replaces op_Linear::forward (cuda_bert/ops/linear.cu:91-148) + op_Gelu /
+ * op_Tanh (ops/elementwise.cu:37-70). */
+int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int M, int N, int K,
+                   int ldx, int elt, int out_elt, int epilogue, int tile, void* stream);
+
+/* Fused QKV projection (op_BatchedLinear::forward, cuda_bert/ops/linear.cu:241-319):
+ * X[B*S, hidden] * Wqkv[3*hidden, hidden]^T + bias -> q,k [B,heads,S,64],
+ * vt [B,heads,64,Sp] with Sp = S rounded up to 32. */
+int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q, void* k, void* vt,
+                       int B, int S, int heads, int elt, int tile, void* stream);
+
+/* Fused attention (Query_Key + op_SoftMax + Prob_Value,
+ * cuda_bert/ops/batch_matmul.cu:48-141, ops/softmax.cu:86-143). */
+int cubert_op_attention(const void* q, const void* k, const void* vt, const float* maskadd,
+                        void* ctx, int B, int heads, int S, float scale, int elt, void* stream);
+
+/* x <- LayerNorm(x + y); optional bf16 copy xb (op_LayerNorm::forward,
+ * cuda_bert/ops/layernorm.cu:136-206). */
+int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
+                            const float* beta, void* xb, int rows, int hidden, void* stream);
+
+/* Embedding gather + add + LayerNorm + additive mask rows (Embedding::forward,
+ * cuda_bert/ops/embedding.cu:3-58). */
+int cubert_op_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
+                              const float* pos, const float* type, const float* gamma,
+                              const float* beta, float* x, void* xb, float* maskadd, int B, int S,
+                              int hidden, int vocab, int type_vocab, void* stream);
+
+/* In-place scale + mask + softmax over materialised scores [B, rows_per_batch, S]
+ * (cuApplySoftmax, cuda_bert/ops/softmax.cu:86-143). */
+int cubert_op_mask_softmax(void* scores, int elt, const int* mask, int B, int rows_per_batch,
+                           int S, float scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUBERT_H_ */

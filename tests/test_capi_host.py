@@ -1,0 +1,153 @@
+"""Host-only checks of the C ABI library: it loads without a GPU, exports every
+symbol include/cubert.h declares, and the weight-directory validation (names,
+dtypes, shapes) rejects what it should -- all without a compute call."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from cudabert_amd import weights as W
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def pb():
+    from cudabert_amd import pybert
+    return pybert
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "cubert.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\([^;{]*\)\s*;", text)))
+
+
+def test_exports_every_declared_symbol(pb):
+    syms = declared_symbols()
+    for must in ("init_model", "release_model", "Cuda_Bert", "Cuda_Inference", "test", "cubert_encode",
+                 "cubert_op_gemm", "cubert_op_attention", "cubert_op_add_layernorm", "cubert_op_mask_softmax"):
+        assert must in syms
+    for s in syms:
+        assert hasattr(pb.lib, s), s
+
+
+def test_reference_argtypes(pb):
+    # cuda_bert/pybert.py:14-38
+    assert pb.init_model.argtypes == [ctypes.c_bool, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_char_p]
+    assert pb.init_model.restype is ctypes.c_void_p
+    assert len(pb.bert.argtypes) == 7 and len(pb.inference.argtypes) == 6
+    assert [f[0] for f in pb.Retval._fields_] == ["tensor", "Pooled_Output"]
+    assert ctypes.sizeof(pb.Retval) == 16
+
+
+@pytest.fixture()
+def tiny_dir(tmp_path):
+    return W.export_npy_dir(W.synth_state(W.TINY, seed=1, degenerate=False), str(tmp_path / "m"))
+
+
+T = W.TINY
+
+
+def chk(pb, d, dims=T):
+    pb.check_weight_dir(d, dims.hidden, dims.layers, dims.heads, dims.inter)
+
+
+def test_valid_dir_accepted(pb, tiny_dir):
+    chk(pb, tiny_dir)
+    # any file-name prefix works, as with the reference's substring lookup (load_model.cc:15-30)
+    for f in os.listdir(tiny_dir):
+        if f.startswith("bert_"):
+            os.rename(os.path.join(tiny_dir, f), os.path.join(tiny_dir, f[len("bert_"):]))
+    chk(pb, tiny_dir)
+
+
+def test_missing_dir_and_empty_dir(pb, tmp_path):
+    with pytest.raises(pb.CubertError, match="cannot open"):
+        chk(pb, str(tmp_path / "nope"))
+    os.makedirs(tmp_path / "empty")
+    with pytest.raises(pb.CubertError, match="no .npy"):
+        chk(pb, str(tmp_path / "empty"))
+
+
+def test_missing_tensor(pb, tiny_dir):
+    os.remove(os.path.join(tiny_dir, "bert_encoder_layer_1_output_dense_bias.npy"))
+    with pytest.raises(pb.CubertError, match="_1_output_dense_bias"):
+        chk(pb, tiny_dir)
+
+
+def test_wrong_dtype(pb, tiny_dir):
+    p = os.path.join(tiny_dir, "bert_pooler_dense_bias.npy")
+    np.save(p, np.load(p).astype(np.float64))
+    with pytest.raises(pb.CubertError, match="float32"):
+        chk(pb, tiny_dir)
+
+
+def test_wrong_shape_and_orientation(pb, tiny_dir):
+    p = os.path.join(tiny_dir, "bert_encoder_layer_0_intermediate_dense_kernel.npy")
+    np.save(p, np.ascontiguousarray(np.load(p).T))            # [out,in] instead of [in,out]
+    with pytest.raises(pb.CubertError, match="intermediate_dense_kernel"):
+        chk(pb, tiny_dir)
+
+
+def test_fortran_order_and_truncation(pb, tiny_dir):
+    p = os.path.join(tiny_dir, "bert_encoder_layer_0_output_dense_kernel.npy")
+    a = np.load(p)
+    np.save(p, np.asfortranarray(a))
+    with pytest.raises(pb.CubertError, match="fortran"):
+        chk(pb, tiny_dir)
+    np.save(p, a)
+    raw = open(p, "rb").read()
+    open(p, "wb").write(raw[:-8])
+    with pytest.raises(pb.CubertError, match="truncated"):
+        chk(pb, tiny_dir)
+
+
+def test_ambiguous_names(pb, tiny_dir):
+    src = os.path.join(tiny_dir, "bert_pooler_dense_kernel.npy")
+    np.save(os.path.join(tiny_dir, "copy_of_bert_pooler_dense_kernel.npy"), np.load(src))
+    with pytest.raises(pb.CubertError, match="more than one"):
+        chk(pb, tiny_dir)
+
+
+def test_dimension_mismatch_and_head_dim(pb, tiny_dir):
+    with pytest.raises(pb.CubertError):
+        pb.check_weight_dir(tiny_dir, 256, T.layers, 4, T.inter)      # wrong hidden
+    with pytest.raises(pb.CubertError, match="64"):
+        pb.check_weight_dir(tiny_dir, T.hidden, T.layers, 4, T.inter)  # head dim 32
+    with pytest.raises(pb.CubertError, match="_2_"):
+        pb.check_weight_dir(tiny_dir, T.hidden, 3, T.heads, T.inter)   # a layer too many
+
+
+def test_npy_versions(pb, tiny_dir):
+    """Format 2.0 headers are accepted (the reference's reader assumed 1.0)."""
+    p = os.path.join(tiny_dir, "bert_pooler_dense_bias.npy")
+    a = np.load(p)
+    with open(p, "wb") as f:
+        np.lib.format.write_array(f, a, version=(2, 0))
+    chk(pb, tiny_dir)
+
+
+def test_init_model_without_gpu_reports_error(pb, tiny_dir):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(pb.CubertError):
+        pb.load_model_ex(tiny_dir, T.hidden, T.layers, T.heads, T.inter)
+
+
+def test_cuda_bert_exits_on_error_like_the_reference():
+    """Cuda_Bert has no error return: an invalid call terminates the process
+    (cuda_bert/utils/manager.cu:100-108, common.h:58-65)."""
+    code = ("import numpy as np\n"
+            "from cudabert_amd import pybert\n"
+            "z = np.zeros((1, 4), np.int32)\n"
+            "pybert.bert(None, np.zeros((1, 8), np.float32), z, z, 1, 4, z)\n"
+            "print('survived')\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
+    assert r.returncode == 1 and "survived" not in r.stdout
+    assert "Cuda_Bert failed" in r.stderr

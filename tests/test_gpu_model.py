@@ -1,0 +1,225 @@
+"""End-to-end parity of the engine (through the C ABI) against the CPU oracle.
+
+Tolerances are the ones the engine is specified to: max-abs 1e-3 for float32
+operands and 3e-2 for bfloat16 operands, on the sequence output and on the
+pooled output.  For bfloat16 the reference checkpoint is made bf16-representable
+first (both sides then hold identical weights); the additional error an
+arbitrary float32 checkpoint picks up from being rounded to bfloat16 storage is
+reported by test_bf16_weight_rounding_cost.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from cudabert_amd import synth
+from cudabert_amd import weights as W
+from oracle import bert_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = 0, 1
+TOL = {F32: 1e-3, BF16: 3e-2}
+
+
+@pytest.fixture(scope="module")
+def pb():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from cudabert_amd import pybert
+    return pybert
+
+
+def bf16_exact(state):
+    out = {}
+    for k, v in state.items():
+        t = torch.from_numpy(v)
+        out[k] = t.to(torch.bfloat16).to(torch.float32).numpy() if v.ndim == 2 and "embeddings" not in k else v
+    return out
+
+
+def load(pb, dims, wdir, precision, maxB, maxS, graph=0):
+    return pb.load_model_ex(wdir, dims.hidden, dims.layers, dims.heads, dims.inter, precision=precision,
+                            max_batchsize=maxB, max_seq_length=maxS, graph_max_tokens=graph)
+
+
+@pytest.fixture(scope="module")
+def tiny_dir(tmp_path_factory):
+    d = tmp_path_factory.mktemp("tiny")
+    state = W.synth_state(W.TINY, seed=7, degenerate=False)
+    W.export_npy_dir(state, str(d / "f32"))
+    W.export_npy_dir(bf16_exact(state), str(d / "bf16"))
+    return d
+
+
+@pytest.mark.parametrize("S", [5, 16, 33])
+def test_tiny_golden_fp32(pb, tiny_dir, golden_dir, S):
+    g = np.load(os.path.join(golden_dir, f"tiny_nd_s{S}.npz"))
+    m = load(pb, W.TINY, str(tiny_dir / "f32"), F32, 4, 64)
+    try:
+        pooled, seq, cls = pb.encode(m, g["ids"], g["seg"], g["mask"], want_seq=True, want_cls=True)
+    finally:
+        pb.unload_model(m)
+    assert np.abs(seq - g["seq"]).max() < TOL[F32]
+    assert np.abs(pooled - g["pooled"]).max() < TOL[F32]
+    npy = W.load_npy_dir(str(tiny_dir / "f32"))
+    assert np.abs(cls - O.classifier_head(npy, g["pooled"])).max() < 1e-4
+
+
+@pytest.mark.parametrize("precision", [F32, BF16])
+def test_tiny_ragged_vs_oracle(pb, tiny_dir, precision):
+    wdir = str(tiny_dir / ("f32" if precision == F32 else "bf16"))
+    npy = W.load_npy_dir(wdir)
+    m = load(pb, W.TINY, wdir, precision, 8, 64)
+    try:
+        for S, lens in ((1, [1]), (7, [7, 1, 4]), (32, [32, 31, 2, 17]), (64, [64, 33, 5, 50, 64, 1, 2, 3])):
+            ids, seg, mask = synth.make_inputs(len(lens), S, lens, vocab=W.TINY.vocab, seed=S, prune=False)
+            seq_ref, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+            pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+            assert np.abs(seq - seq_ref).max() < TOL[precision], (S, np.abs(seq - seq_ref).max())
+            assert np.abs(pooled - pooled_ref).max() < TOL[precision]
+            # mask == NULL is "all valid" (cuda_bert/utils/bert.cu:108-122)
+            seq_ref2, pooled_ref2 = O.forward_torch(npy, W.TINY.heads, ids, seg, None)
+            pooled2, seq2, _ = pb.encode(m, ids, seg, None, want_seq=True)
+            assert np.abs(seq2 - seq_ref2).max() < TOL[precision]
+            assert np.abs(pooled2 - pooled_ref2).max() < TOL[precision]
+    finally:
+        pb.unload_model(m)
+
+
+def test_reference_entry_points(pb, tiny_dir):
+    """Cuda_Bert / Cuda_Inference as the reference's Python calls them
+    (cuda_model.py:23-37, cuda_bert/pybert.py:31-38)."""
+    wdir = str(tiny_dir / "f32")
+    npy = W.load_npy_dir(wdir)
+    m = load(pb, W.TINY, wdir, F32, 4, 32)
+    try:
+        ids, seg, mask = synth.make_inputs(3, 20, [20, 11, 3], vocab=W.TINY.vocab, seed=1, prune=False)
+        seq_ref, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+        out = np.ones((3, W.TINY.hidden), np.float32)
+        pb.bert(m, out, ids, seg, 3, 20, mask)
+        assert np.abs(out - pooled_ref).max() < TOL[F32]
+        ret = pb.inference(m, ids, seg, 3, 20, mask)
+        assert ret.tensor == pb.lib.cubert_seq_ptr(m) and ret.Pooled_Output == pb.lib.cubert_pooled_ptr(m)
+        pb.check(pb.lib.cubert_sync(m))
+        # capacity and range violations come back as errors from the int-returning entry point
+        big = np.zeros((5, 32), np.int32)
+        with pytest.raises(pb.CubertError, match="capacity"):
+            pb.encode(m, big, big, big)
+        bad = ids.copy()
+        bad[1, 2] = W.TINY.vocab
+        with pytest.raises(pb.CubertError, match="vocabulary"):
+            pb.encode(m, bad, seg, mask)
+    finally:
+        pb.unload_model(m)
+
+
+def test_device_inputs_and_graph_replay(pb, tiny_dir):
+    wdir = str(tiny_dir / "f32")
+    npy = W.load_npy_dir(wdir)
+    m = load(pb, W.TINY, wdir, F32, 4, 64, graph=4096)
+    try:
+        H = W.TINY.hidden
+        for rep in range(5):          # eager, capture, replay, replay, replay -- with host work in between
+            for S, lens in ((33, [33, 9, 20]), (16, [16, 2, 7])):
+                ids, seg, mask = synth.make_inputs(3, S, lens, vocab=W.TINY.vocab, seed=rep * 10 + S, prune=False)
+                seq_ref, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+                d = [torch.from_numpy(a).cuda() for a in (ids, seg, mask)]
+                torch.cuda.synchronize()
+                pb.check(pb.lib.cubert_forward_device(m, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), 3, S))
+                pb.check(pb.lib.cubert_sync(m))
+                pooled = torch.empty((3, H), device="cuda")
+                seq = torch.empty((3, S, H), device="cuda")
+                import ctypes
+                hip = ctypes.CDLL("libamdhip64.so")
+                hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+                assert hip.hipMemcpy(pooled.data_ptr(), pb.lib.cubert_pooled_ptr(m), 3 * H * 4, 3) == 0
+                assert hip.hipMemcpy(seq.data_ptr(), pb.lib.cubert_seq_ptr(m), 3 * S * H * 4, 3) == 0
+                assert np.abs(seq.cpu().numpy() - seq_ref).max() < TOL[F32], rep
+                assert np.abs(pooled.cpu().numpy() - pooled_ref).max() < TOL[F32], rep
+        assert pb.lib.cubert_graphs_cached(m) == 2
+    finally:
+        pb.unload_model(m)
+
+
+@pytest.fixture(scope="module")
+def base_dir(tmp_path_factory):
+    d = tmp_path_factory.mktemp("base")
+    state = W.synth_state(W.BASE, seed=20240, degenerate=True)
+    W.export_npy_dir(state, str(d / "f32"))
+    W.export_npy_dir(bf16_exact(state), str(d / "bf16"))
+    return d
+
+
+def test_base_cfg0_fp32_golden_and_oracle(pb, base_dir, golden_dir):
+    """Benchmark configuration 0: BERT-base, B=8, S=128, ragged, float32."""
+    g = np.load(os.path.join(golden_dir, "base_cfg0_slice.npz"))
+    ids, seg, mask = synth.config_inputs(0)
+    m = pb.load_model(False, str(base_dir / "f32"), 0, 8, 128)      # the reference's own init_model path
+    try:
+        assert pb.lib.cubert_precision(m) == F32
+        pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+    finally:
+        pb.unload_model(m)
+    assert np.abs(pooled - g["pooled"]).max() < TOL[F32]
+    assert np.abs(seq[:, ::16, :32] - g["seq_slice"]).max() < TOL[F32]
+    npy = W.load_npy_dir(str(base_dir / "f32"))
+    seq_ref, pooled_ref = O.forward_torch(npy, W.BASE.heads, ids, seg, mask)
+    print("cfg0 fp32 max-abs: seq %.3g pooled %.3g" % (np.abs(seq - seq_ref).max(), np.abs(pooled - pooled_ref).max()))
+    assert np.abs(seq - seq_ref).max() < TOL[F32]
+    assert np.abs(pooled - pooled_ref).max() < TOL[F32]
+
+
+def test_base_cfg0_bf16(pb, base_dir):
+    ids, seg, mask = synth.config_inputs(0)
+    npy = W.load_npy_dir(str(base_dir / "bf16"))
+    seq_ref, pooled_ref = O.forward_torch(npy, W.BASE.heads, ids, seg, mask)
+    m = load(pb, W.BASE, str(base_dir / "bf16"), BF16, 8, 128)
+    try:
+        pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+    finally:
+        pb.unload_model(m)
+    print("cfg0 bf16 max-abs: seq %.3g pooled %.3g" % (np.abs(seq - seq_ref).max(), np.abs(pooled - pooled_ref).max()))
+    assert np.abs(seq - seq_ref).max() < TOL[BF16]
+    assert np.abs(pooled - pooled_ref).max() < TOL[BF16]
+
+
+def test_bf16_weight_rounding_cost(pb, base_dir):
+    """An arbitrary float32 checkpoint run in bf16 mode: the engine's own error
+    stays as above, the rest is what rounding the weights to bfloat16 storage
+    costs any engine.  Checked against the float32 model with a looser bound and
+    printed for the record."""
+    ids, seg, mask = synth.config_inputs(0)
+    npy32 = W.load_npy_dir(str(base_dir / "f32"))
+    seq_ref, pooled_ref = O.forward_torch(npy32, W.BASE.heads, ids, seg, mask)
+    m = load(pb, W.BASE, str(base_dir / "f32"), BF16, 8, 128)
+    try:
+        pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+    finally:
+        pb.unload_model(m)
+    e_seq, e_pool = np.abs(seq - seq_ref).max(), np.abs(pooled - pooled_ref).max()
+    print("cfg0 bf16 on unrounded f32 checkpoint: seq %.3g pooled %.3g" % (e_seq, e_pool))
+    assert e_seq < 6e-2 and e_pool < 3e-2
+
+
+def test_padding_and_permutation_properties(pb, base_dir):
+    """Size-independent properties at BERT-base scale: extra padding columns do
+    not change valid positions (the frontend's pruning assumption, utils.py:3-13)
+    and permuting the batch permutes the outputs."""
+    ids, seg, mask = synth.config_inputs(1, batch=32)
+    B, S = ids.shape
+    m = load(pb, W.BASE, str(base_dir / "bf16"), BF16, 32, 160)
+    try:
+        pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+        pad = lambda a: np.concatenate([a, np.zeros((B, 160 - S), a.dtype)], axis=1)
+        pooled2, seq2, _ = pb.encode(m, pad(ids), pad(seg), pad(mask), want_seq=True)
+        perm = np.random.default_rng(0).permutation(B)
+        pooled3, seq3, _ = pb.encode(m, ids[perm], seg[perm], mask[perm], want_seq=True)
+    finally:
+        pb.unload_model(m)
+    lens = mask.sum(1)
+    for b in range(B):
+        assert np.abs(seq2[b, :lens[b]] - seq[b, :lens[b]]).max() < 2e-3
+    assert np.abs(pooled2 - pooled).max() < 2e-3
+    assert np.array_equal(seq3, seq[perm]) and np.array_equal(pooled3, pooled[perm])
+    assert np.isfinite(seq).all() and np.abs(pooled).max() < 1.0

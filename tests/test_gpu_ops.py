@@ -1,0 +1,252 @@
+"""Parity of every HIP kernel, called through the C ABI on caller-owned device
+memory, against float64/float32 CPU restatements of the same operation."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = 0, 1
+
+
+@pytest.fixture(scope="module")
+def pb():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from cudabert_amd import pybert
+    return pybert
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def bf16_round(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(torch.float32).numpy()
+
+
+def gelu64(x):
+    from scipy.special import erf
+    return x * 0.5 * (1.0 + erf(x / math.sqrt(2.0)))
+
+
+@pytest.mark.parametrize("elt", [F32, BF16])
+@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("M,N,K,epi", [(200, 128, 128, 0), (333, 384, 256, 1), (512, 1024, 1024, 0),
+                                       (77, 512, 512, 2), (1000, 768, 3072, 0)])
+def test_gemm(pb, elt, tile, M, N, K, epi):
+    print("gemm", elt, tile, M, N, K, epi, flush=True)
+    rng = np.random.default_rng(M * 7 + N + K + epi)
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    tdt = torch.float32 if elt == F32 else torch.bfloat16
+    if elt == BF16:
+        X, W = bf16_round(X), bf16_round(W)
+    ref = X.astype(np.float64) @ W.astype(np.float64).T + b
+    if epi == 1:
+        ref = gelu64(ref)
+    elif epi == 2:
+        ref = np.tanh(ref)
+    for out_elt in ([F32] if elt == F32 else [F32, BF16]):
+        Xd, Wd, bd = dev(X, tdt), dev(W, tdt), dev(b)
+        Y = torch.full((M, N), float("nan"), dtype=torch.float32 if out_elt == F32 else torch.bfloat16, device="cuda")
+        pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), M, N, K, K, elt,
+                                       out_elt, epi, tile, stream()))
+        torch.cuda.synchronize()
+        got = Y.float().cpu().numpy().astype(np.float64)
+        tol = 2e-4 if out_elt == F32 else 2e-2 * max(1.0, np.abs(ref).max() / 4)
+        assert np.isfinite(got).all()
+        assert np.abs(got - ref).max() < tol, (elt, out_elt, tile, np.abs(got - ref).max())
+
+
+def test_gemm_strided_rows(pb):
+    """The pooler reads the first token of every sequence: row stride S*H."""
+    rng = np.random.default_rng(5)
+    B, S, H = 6, 9, 128
+    seq = rng.standard_normal((B, S, H)).astype(np.float32)
+    W = (rng.standard_normal((H, H)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(H).astype(np.float32)
+    ref = np.tanh(seq[:, 0].astype(np.float64) @ W.T.astype(np.float64) + b)
+    Xd, Wd, bd = dev(seq), dev(W), dev(b)
+    Y = torch.zeros((B, H), device="cuda")
+    pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), B, H, H, S * H, F32, F32,
+                                   2, 0, stream()))
+    torch.cuda.synchronize()
+    assert np.abs(Y.cpu().numpy() - ref).max() < 1e-4
+
+
+def test_gemm_rejects_bad_shapes(pb):
+    X = torch.zeros((64, 96), device="cuda")
+    W = torch.zeros((64, 96), device="cuda")
+    b = torch.zeros(64, device="cuda")
+    Y = torch.zeros((64, 64), device="cuda")
+    rc = pb.lib.cubert_op_gemm(X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), 64, 64, 96, 96, BF16, F32, 0, 0,
+                               stream())
+    assert rc != 0 and "multiple of 64" in pb.last_error()
+    rc = pb.lib.cubert_op_gemm(X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), 64, 64, 96, 96, F32, F32, 0, 99,
+                               stream())
+    assert rc != 0
+
+
+@pytest.mark.parametrize("elt", [F32, BF16])
+@pytest.mark.parametrize("B,S,heads,tile", [(3, 33, 2, 64), (2, 200, 4, 128), (5, 128, 12, 256)])
+def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile):
+    print("qkv", elt, B, S, heads, tile, flush=True)
+    rng = np.random.default_rng(B + S)
+    H = heads * 64
+    Sp = (S + 31) // 32 * 32
+    X = rng.standard_normal((B * S, H)).astype(np.float32)
+    W = (rng.standard_normal((3 * H, H)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(3 * H).astype(np.float32)
+    tdt = torch.float32 if elt == F32 else torch.bfloat16
+    if elt == BF16:
+        X, W = bf16_round(X), bf16_round(W)
+    y = (X.astype(np.float64) @ W.T.astype(np.float64) + b).reshape(B, S, 3, heads, 64)
+    q_ref = y[:, :, 0].transpose(0, 2, 1, 3)             # [B, heads, S, 64]
+    k_ref = y[:, :, 1].transpose(0, 2, 1, 3)
+    vt_ref = y[:, :, 2].transpose(0, 2, 3, 1)            # [B, heads, 64, S]
+    Xd, Wd, bd = dev(X, tdt), dev(W, tdt), dev(b)
+    q = torch.zeros((B, heads, S, 64), dtype=tdt, device="cuda")
+    k = torch.zeros_like(q)
+    vt = torch.zeros((B, heads, 64, Sp), dtype=tdt, device="cuda")
+    pb.check(pb.lib.cubert_op_gemm_qkv(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), q.data_ptr(), k.data_ptr(),
+                                       vt.data_ptr(), B, S, heads, elt, tile, stream()))
+    torch.cuda.synchronize()
+    tol = 2e-4 if elt == F32 else 3e-2
+    assert np.abs(q.float().cpu().numpy() - q_ref).max() < tol
+    assert np.abs(k.float().cpu().numpy() - k_ref).max() < tol
+    vt_h = vt.float().cpu().numpy()
+    assert np.abs(vt_h[..., :S] - vt_ref).max() < tol
+    assert (vt_h[..., S:] == 0).all()                    # padding columns untouched
+
+
+@pytest.mark.parametrize("elt", [F32, BF16])
+@pytest.mark.parametrize("B,S,heads", [(2, 5, 2), (3, 33, 2), (2, 200, 3), (1, 512, 2), (4, 128, 12)])
+def test_attention(pb, elt, B, S, heads):
+    print("attention", elt, B, S, heads, flush=True)
+    rng = np.random.default_rng(S * 3 + B)
+    Sp = (S + 31) // 32 * 32
+    q = rng.standard_normal((B, heads, S, 64)).astype(np.float32)
+    k = rng.standard_normal((B, heads, S, 64)).astype(np.float32)
+    v = rng.standard_normal((B, heads, S, 64)).astype(np.float32)
+    lens = rng.integers(1, S + 1, size=B)
+    lens[0] = S
+    mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.float32)
+    tdt = torch.float32 if elt == F32 else torch.bfloat16
+    if elt == BF16:
+        q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
+    scale = 1.0 / 8.0
+    sc = np.einsum("bhsd,bhtd->bhst", q.astype(np.float64), k.astype(np.float64)) * scale
+    sc = sc + ((1.0 - mask) * -10000.0)[:, None, None, :]
+    sc = sc - sc.max(-1, keepdims=True)
+    p = np.exp(sc)
+    p /= p.sum(-1, keepdims=True)
+    ref = np.einsum("bhst,bhtd->bshd", p, v.astype(np.float64)).reshape(B * S, heads * 64)
+    vt = np.zeros((B, heads, 64, Sp), np.float32)
+    vt[..., :S] = v.transpose(0, 1, 3, 2)
+    maskadd = np.full((B, Sp), -np.inf, np.float32)
+    maskadd[:, :S] = (1.0 - mask) * -10000.0
+    qd, kd, vd, md = dev(q, tdt), dev(k, tdt), dev(vt, tdt), dev(maskadd)
+    ctx = torch.full((B * S, heads * 64), float("nan"), dtype=tdt, device="cuda")
+    pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), ctx.data_ptr(),
+                                        B, heads, S, scale, elt, stream()))
+    torch.cuda.synchronize()
+    got = ctx.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    tol = 2e-5 * 10 if elt == F32 else 2e-2
+    assert np.abs(got - ref).max() < tol, np.abs(got - ref).max()
+
+
+@pytest.mark.parametrize("H", [128, 768, 1024])
+@pytest.mark.parametrize("y_elt", [None, F32, BF16])
+def test_add_layernorm(pb, H, y_elt):
+    rng = np.random.default_rng(H)
+    rows = 1001
+    x = (rng.standard_normal((rows, H)) * 2 + 0.5).astype(np.float32)
+    y = rng.standard_normal((rows, H)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(H)).astype(np.float32)
+    if y_elt == BF16:
+        y = bf16_round(y)
+    s = x.astype(np.float64) + (y if y_elt is not None else 0.0)
+    u = s.mean(-1, keepdims=True)
+    var = ((s - u) ** 2).mean(-1, keepdims=True)
+    ref = g * ((s - u) / np.sqrt(var + 1e-12)) + b
+    xd, gd, bd = dev(x), dev(g), dev(b)
+    yd = None if y_elt is None else dev(y, torch.float32 if y_elt == F32 else torch.bfloat16)
+    xb = torch.zeros((rows, H), dtype=torch.bfloat16, device="cuda")
+    pb.check(pb.lib.cubert_op_add_layernorm(xd.data_ptr(), None if yd is None else yd.data_ptr(), y_elt or 0,
+                                            gd.data_ptr(), bd.data_ptr(), xb.data_ptr(), rows, H, stream()))
+    torch.cuda.synchronize()
+    got = xd.cpu().numpy()
+    assert np.abs(got - ref).max() < 2e-5
+    assert np.array_equal(xb.float().cpu().numpy(), bf16_round(got))     # bf16 copy is the RNE of the f32 result
+
+
+def test_embed_layernorm(pb):
+    rng = np.random.default_rng(11)
+    B, S, H, V = 3, 37, 768, 500
+    Sp = 64
+    word = rng.standard_normal((V, H)).astype(np.float32)
+    pos = rng.standard_normal((64, H)).astype(np.float32)
+    typ = rng.standard_normal((2, H)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(H)).astype(np.float32)
+    ids = rng.integers(0, V, size=(B, S)).astype(np.int32)
+    seg = rng.integers(0, 2, size=(B, S)).astype(np.int32)
+    mask = (rng.random((B, S)) < 0.7).astype(np.int32)
+    e = word[ids].astype(np.float64) + pos[np.arange(S)][None] + typ[seg]
+    u = e.mean(-1, keepdims=True)
+    var = ((e - u) ** 2).mean(-1, keepdims=True)
+    ref = g * ((e - u) / np.sqrt(var + 1e-12)) + b
+    x = torch.zeros((B * S, H), device="cuda")
+    xb = torch.zeros((B * S, H), dtype=torch.bfloat16, device="cuda")
+    madd = torch.zeros((B, Sp), device="cuda")
+    args = [dev(a) for a in (ids, seg, mask, word, pos, typ, g, b)]
+    pb.check(pb.lib.cubert_op_embed_layernorm(*[a.data_ptr() for a in args], x.data_ptr(), xb.data_ptr(),
+                                              madd.data_ptr(), B, S, H, V, 2, stream()))
+    torch.cuda.synchronize()
+    got = x.cpu().numpy().reshape(B, S, H)
+    assert np.abs(got - ref).max() < 2e-5
+    m = madd.cpu().numpy()
+    assert np.array_equal(m[:, :S], (1.0 - mask) * np.float32(-10000.0))
+    assert np.isneginf(m[:, S:]).all()
+    # mask == NULL: everything valid
+    pb.check(pb.lib.cubert_op_embed_layernorm(args[0].data_ptr(), args[1].data_ptr(), None,
+                                              *[a.data_ptr() for a in args[3:]], x.data_ptr(), None,
+                                              madd.data_ptr(), B, S, H, V, 2, stream()))
+    torch.cuda.synchronize()
+    assert (madd.cpu().numpy()[:, :S] == 0).all()
+
+
+@pytest.mark.parametrize("elt", [F32, BF16])
+@pytest.mark.parametrize("B,R,S", [(2, 6, 5), (3, 2 * 33, 33), (2, 4 * 200, 200), (1, 512, 512)])
+def test_mask_softmax(pb, elt, B, R, S):
+    rng = np.random.default_rng(S)
+    sc = (rng.standard_normal((B, R, S)) * 3).astype(np.float32)
+    mask = (rng.random((B, S)) < 0.6).astype(np.int32)
+    mask[:, 0] = 1
+    tdt = torch.float32 if elt == F32 else torch.bfloat16
+    if elt == BF16:
+        sc = bf16_round(sc)
+    z = sc.astype(np.float64) * 0.125 + ((1.0 - mask) * -10000.0)[:, None, :]
+    z = z - z.max(-1, keepdims=True)
+    p = np.exp(z)
+    ref = p / p.sum(-1, keepdims=True)
+    d = dev(sc, tdt)
+    md = dev(mask)
+    pb.check(pb.lib.cubert_op_mask_softmax(d.data_ptr(), elt, md.data_ptr(), B, R, S, 0.125, stream()))
+    torch.cuda.synchronize()
+    got = d.float().cpu().numpy()
+    assert np.abs(got - ref).max() < (1e-6 if elt == F32 else 4e-3)
+    assert np.abs(got.sum(-1) - 1).max() < (1e-5 if elt == F32 else 2e-2)
+    assert (got[np.broadcast_to(mask[:, None, :] == 0, got.shape)] == 0).all()
