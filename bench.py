@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Throughput benchmark of the encoder hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision bf16|fp32]
+                    [--config 2] [--no-cpu]
+
+A step is one forward pass (embedding -> 24 layers -> pooler -> classifier head)
+over one synthetic batch of the headline configuration: BERT-large, batch 128,
+seq 200, per-row valid lengths uniform in [100, 200], stock N(0, 0.02) weights.
+Inputs are resident in device memory when the timed region starts.  Prints one
+JSON line with the whole-job rate, the roofline figure of the dominant kernel
+(the FFN GEMM, timed with HIP events around back-to-back launches on the stream
+they are launched on), a per-phase breakdown with achieved TFLOP/s and GB/s,
+and the CPU oracle's rate on a bounded sample of the same batch.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+PEAK_HBM_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--precision", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 4])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seqs", type=int, default=128, help="sequences in the CPU baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU; --gpus %d is not supported (every replica of the "
+              "encoder is independent, so more GPUs are more processes of this same run)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from cudabert_amd import pybert, synth
+    from cudabert_amd import weights as W
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    large, B, S0 = synth.CONFIG_SHAPES[args.config]
+    dims = W.LARGE if large else W.BASE
+    prec = pybert.BF16 if args.precision == "bf16" else pybert.F32
+    ids, seg, mask = synth.config_inputs(args.config)
+    B, S = ids.shape
+    N = B * S
+    H, I, L, A = dims.hidden, dims.inter, dims.layers, dims.heads
+    es = 2 if prec == pybert.BF16 else 4
+
+    t0 = time.time()
+    state = W.synth_state(dims, seed=20240, degenerate=True)
+    npy = W.to_npy_layout(state)
+    del state
+    with tempfile.TemporaryDirectory(prefix="cubert_w_") as wdir:
+        for name, arr in npy.items():
+            np.save(os.path.join(wdir, name + ".npy"), arr)
+        t_gen = time.time() - t0
+        t0 = time.time()
+        model = pybert.load_model_ex(wdir, H, L, A, I, precision=prec, max_batchsize=B, max_seq_length=S,
+                                     graph_max_tokens=0)
+        t_load = time.time() - t0
+    lib = pybert.lib
+    d_ids, d_seg, d_mask = (torch.from_numpy(a).cuda() for a in (ids, seg, mask))
+    torch.cuda.synchronize()
+
+    def step():
+        pybert.check(lib.cubert_forward_device(model, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S))
+        pybert.check(lib.cubert_classify(model))
+
+    for _ in range(args.warmup):
+        step()
+    pybert.check(lib.cubert_sync(model))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    pybert.check(lib.cubert_sync(model))
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = B * args.steps / elapsed
+
+    # ---- per-phase breakdown (events before every launch; outside the timed region) ----
+    ph = (ctypes.c_float * 8)()
+    acc = np.zeros(8)
+    reps = 3
+    for _ in range(reps):
+        pybert.check(lib.cubert_profile_device(model, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S, ph))
+        acc += np.array(list(ph))
+    acc /= reps
+    gf = {"qkv_gemm": 2.0 * N * H * 3 * H * L, "attn_out_gemm": 2.0 * N * H * H * L,
+          "ffn_in_gemm": 2.0 * N * H * I * L, "ffn_out_gemm": 2.0 * N * I * H * L,
+          "attention": 4.0 * N * S * H * L, "pooler": 2.0 * B * H * H}
+    # residual+LayerNorm traffic as executed: x f32 read + y f32 read + x f32 write (+ bf16 copy)
+    ln_bytes_alg = (3.0 * N * H * 4 + 2 * H * 4) * 2 * L
+    ln_bytes_exec = ((3 * 4 + (2 if prec == pybert.BF16 else 0)) * N * H + 2 * H * 4) * 2 * L
+    emb_bytes = N * (12 + H * 4 + H * 4) + (S + 2) * H * 4 + 2 * H * 4
+    phases = {}
+    for i, name in enumerate(pybert.PHASES):
+        ms = float(acc[i])
+        e = {"ms": round(ms, 4)}
+        if name in gf and ms > 0:
+            e["tflops"] = round(gf[name] / ms / 1e9, 1)
+            e["frac_mfma_peak"] = round(e["tflops"] / PEAK_TFLOPS[args.precision], 4)
+        if name == "add_layernorm" and ms > 0:
+            e["gbs_algorithmic"] = round(ln_bytes_alg / ms / 1e6, 1)
+            e["gbs_executed"] = round(ln_bytes_exec / ms / 1e6, 1)
+            e["frac_hbm_peak"] = round(e["gbs_executed"] / PEAK_HBM_GBS, 4)
+        if name == "embedding" and ms > 0:
+            e["gbs_algorithmic"] = round(emb_bytes / ms / 1e6, 1)
+        phases[name] = e
+    gemm_ms = sum(acc[i] for i, n in enumerate(pybert.PHASES) if n.endswith("_gemm"))
+    gemm_flops = sum(gf[n] for n in gf if n.endswith("_gemm"))
+    phases["all_gemms"] = {"ms": round(float(gemm_ms), 3), "tflops": round(gemm_flops / gemm_ms / 1e9, 1),
+                           "frac_mfma_peak": round(gemm_flops / gemm_ms / 1e9 / PEAK_TFLOPS[args.precision], 4)}
+
+    # ---- roofline of the dominant kernel: the FFN-in GEMM (bias+GELU epilogue) ----
+    tdt = torch.bfloat16 if prec == pybert.BF16 else torch.float32
+    X = (torch.randn((N, H), device="cuda") * 1.0).to(tdt)
+    Wt = (torch.randn((I, H), device="cuda") * 0.02).to(tdt)
+    bias = torch.zeros(I, device="cuda")
+    Y = torch.empty((N, I), dtype=tdt, device="cuda")
+    st = torch.cuda.current_stream()
+    out_elt = prec
+
+    def ffn_in():
+        pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H, prec,
+                                        out_elt, 1, 0, st.cuda_stream))
+    for _ in range(3):
+        ffn_in()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    launches = 20
+    e0.record(st)
+    for _ in range(launches):
+        ffn_in()
+    e1.record(st)
+    e1.synchronize()
+    k_ms = e0.elapsed_time(e1) / launches
+    flops_per_launch = 2.0 * N * H * I
+    achieved = flops_per_launch / k_ms / 1e9
+    roofline = {"bound": "mfma", "kernel": "gemm_kernel<%s, bias+GELU, tile 256> (FFN-in %dx%dx%d)" %
+                (args.precision, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[args.precision],
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[args.precision], 4),
+                "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch, "traffic": None}
+    del X, Wt, Y
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same batch ----
+    cpu = None
+    if not args.no_cpu:
+        from oracle import bert_oracle as O
+        n = min(args.cpu_seqs, B)
+        cores = os.cpu_count() or 1
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+        torch.set_num_threads(cores)
+        O.forward_torch(npy, A, ids[:1], seg[:1], mask[:1])         # warm-up (thread pool, allocator)
+        t0 = time.perf_counter()
+        seq_ref, pooled_ref = O.forward_torch(npy, A, ids[:n], seg[:n], mask[:n])
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(n / dt, 3), "unit": "sequences/s", "cores": cores, "kind": "port",
+               "sample": "first %d sequences of the same batch (S=%d), fp32 torch oracle, 1 pass, %.1f s" % (n, S, dt)}
+        # the sample doubles as a full-size parity spot check
+        pooled = torch.empty((B, H), device="cuda")
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        step()
+        pybert.check(lib.cubert_sync(model))
+        assert hip.hipMemcpy(pooled.data_ptr(), lib.cubert_pooled_ptr(model), B * H * 4, 3) == 0
+        cpu["pooled_max_abs_vs_gpu"] = float(np.abs(pooled.cpu().numpy()[:n] - pooled_ref).max())
+    pybert.unload_model(model)
+
+    out = {
+        "metric": "sequences/s BERT-large b128 s200 on 1 MI355X" if args.config == 2 else
+                  "sequences/s cfg%d on 1 MI355X" % args.config,
+        "value": round(value, 2), "unit": "sequences/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.precision, "data": "synthetic",
+        "config": {"workload": "cfg%d: BERT-%s encoder + pooler + Linear(H->2)+softmax head, batch %d, seq %d "
+                               "(valid lengths ragged, pruned to batch max), inputs resident in HBM" %
+                               (args.config, "large" if large else "base", B, S),
+                   "batch": B, "seq_len": S, "tokens": N, "precision": args.precision},
+        "roofline": roofline, "cpu_baseline": cpu, "phases": phases,
+        "gemm_tflop_per_step": round(gemm_flops / 1e12, 3),
+        "setup_s": {"weights_generate_write": round(t_gen, 1), "model_load": round(t_load, 1)},
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -142,6 +142,22 @@ int cubert_forward_device(void* model, const int* d_words, const int* d_token_ty
     return m->forward_device(d_words, d_token_types, d_attention_mask, batchsize, seq_length) ? 0 : 1;
 }
 
+int cubert_classify(void* model) {
+    cubert::set_error("");
+    Model* m = as_model(model, "cubert_classify");
+    return (m && m->classify()) ? 0 : 1;
+}
+
+float* cubert_cls_ptr(void* model) { return model ? static_cast<Model*>(model)->cls_ptr() : nullptr; }
+
+int cubert_profile_device(void* model, const int* d_words, const int* d_token_types, const int* d_attention_mask,
+                          int batchsize, int seq_length, float* phase_ms) {
+    cubert::set_error("");
+    Model* m = as_model(model, "cubert_profile_device");
+    if (!m) return 1;
+    return m->profile_device(d_words, d_token_types, d_attention_mask, batchsize, seq_length, phase_ms) ? 0 : 1;
+}
+
 int cubert_sync(void* model) {
     Model* m = as_model(model, "cubert_sync");
     return (m && m->sync()) ? 0 : 1;

@@ -41,6 +41,7 @@ Model::~Model() {
     if (stream_) (void)hipStreamSynchronize(stream_);
     for (auto& kv : graphs_)
         if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+    for (hipEvent_t e : prof_events_) (void)hipEventDestroy(e);
     if (wblock_) (void)hipFree(wblock_);
     if (ablock_) (void)hipFree(ablock_);
     if (h_in_) (void)hipHostFree(h_in_);
@@ -286,6 +287,7 @@ bool Model::enqueue(int B, int S, bool has_mask) {
     const void* xin = elt == kBF16 ? static_cast<const void*>(xb_) : static_cast<const void*>(x32_);
     const float scale = 1.0f / std::sqrt(64.0f);
 
+    if (!mark(kPhEmbed)) return false;
     if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32_, xb_, maskadd_, B, S, Sp, H,
                                 D.vocab, D.type_vocab, stream_))
         return false;
@@ -296,30 +298,74 @@ bool Model::enqueue(int B, int S, bool has_mask) {
         // QKV projection, scattered per head (V transposed)
         g.X = xin; g.ldx = H; g.W = L.w_qkv; g.bias = L.b_qkv; g.M = N; g.N = 3 * H; g.K = H;
         g.epilogue = kEpiQKV; g.q = q_; g.k = k_; g.vt = vt_; g.S = S; g.Sp = Sp; g.heads = D.heads;
-        if (!launch_gemm(g, stream_)) return false;
+        if (!mark(kPhQKV) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhAttention)) return false;
         if (!launch_attention(q_, k_, vt_, maskadd_, ctx_, B, D.heads, S, Sp, scale, elt, stream_)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx_; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32_;
         g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias;
-        if (!launch_gemm(g, stream_)) return false;
+        if (!mark(kPhAttnOut) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhLayerNorm)) return false;
         if (!launch_add_layernorm(x32_, y32_, kF32, L.g1, L.be1, xb_, N, H, stream_)) return false;
         // feed-forward
         g = GemmParams();
         g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h_;
         g.M = N; g.N = I; g.K = H; g.epilogue = kEpiBiasGelu;
-        if (!launch_gemm(g, stream_)) return false;
+        if (!mark(kPhFFNIn) || !launch_gemm(g, stream_)) return false;
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = h_; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32_;
         g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias;
-        if (!launch_gemm(g, stream_)) return false;
+        if (!mark(kPhFFNOut) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhLayerNorm)) return false;
         if (!launch_add_layernorm(x32_, y32_, kF32, L.g2, L.be2, xb_, N, H, stream_)) return false;
     }
     // pooler: tanh(dense(first token)); the first-token gather is the row stride S*H
     GemmParams g;
     g.elt = elt; g.out_elt = kF32; g.X = xin; g.ldx = S * H; g.W = w_pool_; g.bias = b_pool_; g.Y = pooled_;
     g.M = B; g.N = H; g.K = H; g.epilogue = kEpiBiasTanh;
+    if (!mark(kPhPooler)) return false;
     return launch_gemm(g, stream_);
+}
+
+bool Model::mark(int phase) {
+    if (!profiling_) return true;
+    if (prof_used_ == prof_events_.size()) {
+        hipEvent_t e;
+        CUBERT_HIP_OK(hipEventCreate(&e));
+        prof_events_.push_back(e);
+    }
+    CUBERT_HIP_OK(hipEventRecord(prof_events_[prof_used_], stream_));
+    if (phase >= 0) prof_phase_.push_back(phase);
+    ++prof_used_;
+    return true;
+}
+
+bool Model::profile_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S, float* phase_ms) {
+    if (!phase_ms) { set_error("profile: null output"); return false; }
+    if (!check_shape(B, S)) return false;
+    if (!d_ids || !d_seg) { set_error("input_ids and token_type_ids must not be null"); return false; }
+    const size_t n = (size_t)B * S, cap = (size_t)cap_tokens_;
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_, d_ids, n * 4, hipMemcpyDeviceToDevice, stream_));
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + cap, d_seg, n * 4, hipMemcpyDeviceToDevice, stream_));
+    if (d_mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, d_mask, n * 4, hipMemcpyDeviceToDevice, stream_));
+    B_ = B;
+    S_ = S;
+    profiling_ = true;
+    prof_used_ = 0;
+    prof_phase_.clear();
+    bool ok = enqueue(B, S, d_mask != nullptr);
+    ok = ok && mark(-1);                       // closing event
+    profiling_ = false;
+    if (!ok) return false;
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    for (int i = 0; i < kNumPhases; ++i) phase_ms[i] = 0.0f;
+    for (size_t i = 0; i + 1 < prof_used_; ++i) {
+        float ms = 0.0f;
+        CUBERT_HIP_OK(hipEventElapsedTime(&ms, prof_events_[i], prof_events_[i + 1]));
+        phase_ms[prof_phase_[i]] += ms;
+    }
+    return true;
 }
 
 bool Model::classify() {

@@ -43,6 +43,11 @@ class Model {
     bool forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S);
     // softmax(pooled @ classifier_kernel + bias) for the last forward -> cls_probs().
     bool classify();
+    // One eager forward pass with a hipEvent before every launch; fills
+    // phase_ms[kNumPhases] with the summed time per phase (milliseconds).
+    enum Phase { kPhEmbed = 0, kPhQKV, kPhAttention, kPhAttnOut, kPhLayerNorm, kPhFFNIn, kPhFFNOut, kPhPooler,
+                 kNumPhases };
+    bool profile_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S, float* phase_ms);
     bool sync();
     bool copy_pooled(float* host_out);                 // D2H + sync, B*hidden floats
     bool copy_seq(float* host_out);                    // D2H + sync, B*S*hidden floats
@@ -68,6 +73,7 @@ class Model {
     bool check_shape(int B, int S);
     bool run(int B, int S, bool has_mask);             // graph or eager
     bool enqueue(int B, int S, bool has_mask);         // the launch sequence
+    bool mark(int phase);                              // profiling: event before a launch
 
     ModelOptions opt_;
     hipStream_t stream_ = nullptr;
@@ -96,6 +102,10 @@ class Model {
     int B_ = 0, S_ = 0;
     struct GraphEntry { hipGraphExec_t exec = nullptr; int seen = 0; };
     std::map<long, GraphEntry> graphs_;
+    bool profiling_ = false;
+    std::vector<hipEvent_t> prof_events_;
+    std::vector<int> prof_phase_;
+    size_t prof_used_ = 0;
 };
 
 }  // namespace cubert

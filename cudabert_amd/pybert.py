@@ -67,6 +67,14 @@ lib.cubert_encode.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_i
 lib.cubert_encode.restype = c_int
 lib.cubert_forward_device.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int]
 lib.cubert_forward_device.restype = c_int
+lib.cubert_classify.argtypes = [c_void_p]
+lib.cubert_classify.restype = c_int
+lib.cubert_cls_ptr.argtypes = [c_void_p]
+lib.cubert_cls_ptr.restype = c_void_p
+lib.cubert_profile_device.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, POINTER(c_float)]
+lib.cubert_profile_device.restype = c_int
+PHASES = ("embedding", "qkv_gemm", "attention", "attn_out_gemm", "add_layernorm", "ffn_in_gemm", "ffn_out_gemm",
+          "pooler")
 lib.cubert_sync.argtypes = [c_void_p]
 lib.cubert_sync.restype = c_int
 lib.cubert_seq_ptr.argtypes = [c_void_p]

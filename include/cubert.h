@@ -104,6 +104,20 @@ int cubert_forward_device(void* model, const int* d_words, const int* d_token_ty
                           const int* d_attention_mask, int batchsize, int seq_length);
 int cubert_sync(void* model);
 
+/* Enqueues the fine-tune head on the pooled output of the last forward pass
+ * (softmax(pooled @ classifier_kernel + bias), apps/finetune.py:16-44; the
+ * reference's commented-out classify_inference, cuda_bert/utils/bert.cu:254-265).
+ * Result: cubert_cls_ptr, device [B, num_classes] float32. */
+int cubert_classify(void* model);
+float* cubert_cls_ptr(void* model);
+
+/* One eager forward pass on device inputs with a hipEvent before every kernel;
+ * phase_ms[8] receives milliseconds summed per phase in the order: embedding,
+ * QKV GEMM, attention, attention-output GEMM, residual+LayerNorm (both per
+ * layer), FFN-in GEMM, FFN-out GEMM, pooler.  Synchronous. */
+int cubert_profile_device(void* model, const int* d_words, const int* d_token_types,
+                          const int* d_attention_mask, int batchsize, int seq_length, float* phase_ms);
+
 /* Introspection. */
 float* cubert_seq_ptr(void* model);       /* device, [B, S, hidden] float32 */
 float* cubert_pooled_ptr(void* model);    /* device, [B, hidden] float32 */
