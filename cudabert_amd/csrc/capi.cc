@@ -242,6 +242,7 @@ int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int
     cubert::GemmParams p;
     p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.elt = elt;
     p.out_elt = out_elt; p.epilogue = epilogue; p.tile = tile;
+    if (tile == 257) { p.tile = 256; p.compiler_scheduled = true; }   // 256 tile, generic (compiler-scheduled) kernel
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
@@ -253,6 +254,7 @@ int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q,
     p.X = X; p.W = W; p.bias = bias; p.M = B * S; p.N = 3 * heads * 64; p.K = heads * 64; p.ldx = heads * 64;
     p.elt = elt; p.epilogue = cubert::kEpiQKV; p.q = q; p.k = k; p.vt = vt; p.S = S; p.Sp = cubert::round_up(S, 32);
     p.heads = heads; p.tile = tile;
+    if (tile == 257) { p.tile = 256; p.compiler_scheduled = true; }
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 

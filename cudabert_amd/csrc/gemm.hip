@@ -3,8 +3,9 @@
 // Both operands are K-contiguous ([rows, K]); a workgroup of four wave64s
 // computes a BT x BT macro tile (BT features x BT tokens), each wave a
 // (BT/2) x (BT/2) quadrant built from 32x32 MFMA blocks.  Per K step a slab of
-// 128 bytes per row (64 bf16 / 32 f32) of both operands is staged through LDS
-// (double buffered, one barrier per step).  LDS rows are 128 bytes = eight
+// 128 bytes per row (64 bf16 / 32 f32) of both operands is loaded straight
+// from global memory into LDS (buffer_load ... lds, double buffered, one
+// barrier per step).  LDS rows are 128 bytes = eight
 // 16-byte chunks; chunk c of row r lives at position c ^ ((r ^ (r >> 3)) & 7)
 // so that the 16-byte fragment reads of 8 (or 16) consecutive rows hit
 // distinct banks.
@@ -19,94 +20,65 @@
 // the 16-byte chunk 2*kk + g of its row for both operands, so A and B always
 // pair identical k.  For f32 each chunk holds four k values consumed by four
 // 32x32x2 MFMAs; for bf16 it holds eight consumed by one 32x32x16 MFMA.
-#include "kernels.h"
+#include <type_traits>
+
+#include "gemm_common.h"
 
 namespace cubert {
+
+bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
+
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+using namespace gemm_detail;
 
-struct GemmDev {
-    const unsigned char* X;
-    const unsigned char* W;
-    const float* bias;
-    unsigned char* Y;
-    unsigned char* q;
-    unsigned char* k;
-    unsigned char* vt;
-    int M, N, K, ldx;
-    int S, Sp, heads, hidden;
-    int tiles_n, tiles_m;
-};
-
-__device__ __forceinline__ float gelu_erf(float x) {
-    return x * 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
-}
-
-template <int ELT>
-__device__ __forceinline__ void mfma_chunk(const u32x4_t& a, const u32x4_t& b, f32x16_t& acc) {
-    if constexpr (ELT == kBF16) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                      __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
-    } else {
-        const f32x4_t fa = __builtin_bit_cast(f32x4_t, a);
-        const f32x4_t fb = __builtin_bit_cast(f32x4_t, b);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1], fb[1], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2], fb[2], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[3], fb[3], acc, 0, 0, 0);
+// Instruction order of one K step, prescribed to the machine scheduler: the
+// fragment reads of k-step 0 first, then per k-step groups of MFMAs with the
+// fragment reads of the following k-step (and, during k-step 0, the
+// global->LDS loads of the next tile) slotted in between, so that LDS and
+// memory latency run under MFMA issue instead of in front of it.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
     }
 }
 
-template <int OUT>
-__device__ __forceinline__ void store4(unsigned char* base, size_t elem_index, const float v[4]) {
-    if constexpr (OUT == kBF16) {
-        bf16x4_t o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-        *reinterpret_cast<bf16x4_t*>(base + elem_index * 2) = o;
-    } else {
-        f32x4_t o = {v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<f32x4_t*>(base + elem_index * 4) = o;
-    }
-}
-
-template <int OUT>
-__device__ __forceinline__ void store1(unsigned char* base, size_t elem_index, float v) {
-    if constexpr (OUT == kBF16) {
-        *reinterpret_cast<__bf16*>(base + elem_index * 2) = (__bf16)v;
-    } else {
-        *reinterpret_cast<float*>(base + elem_index * 4) = v;
-    }
-}
-
-// Workgroup id -> (tile_n, tile_m).  Hardware hands consecutive workgroup ids
-// to the eight XCDs round-robin; the remap gives every XCD one contiguous run
-// of the tile sequence so tiles sharing operand rows share an L2.
-__device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int* tn, int* tm) {
-    const int xcd = pid & 7, idx = pid >> 3;
-    const int base = total >> 3, rem = total & 7;
-    const int start = xcd * base + (xcd < rem ? xcd : rem);
-    const int t = start + idx;
-    *tm = t / tiles_n;
-    *tn = t - *tm * tiles_n;
+template <int NB, int MPC>
+__device__ __forceinline__ void schedule_k_step() {
+    constexpr int RPP = NB == 4 ? 8 : (NB == 2 ? 4 : 1);      // groups per k-step
+    constexpr int MFMA_PER_GROUP = NB * NB * MPC / RPP;
+    constexpr int VMEM_PER_GROUP = 4 * NB / RPP;
+    constexpr int READS_PER_GROUP = 2 * NB / RPP;
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
+    static_for<4>([&](auto ph) {
+        static_for<RPP>([&](auto) {
+            __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER_GROUP, 0);
+            if constexpr (decltype(ph)::value == 0) __builtin_amdgcn_sched_group_barrier(0x010, VMEM_PER_GROUP, 0);
+            if constexpr (decltype(ph)::value < 3) __builtin_amdgcn_sched_group_barrier(0x100, READS_PER_GROUP, 0);
+        });
+    });
 }
 
 template <int ELT, int OUT, int EPI, int BT>
 __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     constexpr int ES = (ELT == kBF16) ? 2 : 4;       // operand element size
     constexpr int NB = BT / 64;                      // 32x32 blocks per wave and dimension
-    constexpr int PASSES = BT / 32;                  // 32 tile rows are loaded per pass
+    constexpr int GROUPS = BT / 32;                  // 8-row groups each wave moves per operand tile
     constexpr int TILE_BYTES = BT * 128;             // one operand tile in LDS
     constexpr int BK = 128 / ES;                     // K elements per step
+    constexpr int MPC = (ELT == kBF16) ? 1 : 4;      // MFMA instructions per 16-byte chunk pair
 
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // Two separate LDS objects (not one array indexed by parity): the compiler
+    // then knows that the asynchronous global->LDS loads filling one buffer
+    // cannot alias the fragment reads of the other and does not serialise them.
+    __shared__ __attribute__((aligned(1024))) unsigned char lds0[2 * TILE_BYTES];   // W tile, then X tile
+    __shared__ __attribute__((aligned(1024))) unsigned char lds1[2 * TILE_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // wave-uniform: keeps LDS bases scalar
     const int wn = wave >> 1, wm = wave & 1;
     const int l32 = lane & 31, g = lane >> 5;
 
@@ -114,46 +86,51 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, &tile_n, &tile_m);
     const int n0 = tile_n * BT, m0 = tile_m * BT;
 
-    // ---- global -> register staging through buffer resources ----
-    // Out-of-range rows (edge tiles) read as zero: the hardware bounds check of
-    // the buffer descriptor replaces per-row clamping.  The check covers the
-    // lane offset only, so the row part lives there and just the K offset
+    // ---- global -> LDS, asynchronous, no registers in between ----
+    // One buffer_load ... lds instruction moves 64 lanes x 16 bytes = 8 tile rows
+    // to 1 KiB of consecutive LDS (lane l lands at base + 16 l).  Wave w moves
+    // the 8-row groups w, w+4, w+8, ...  The LDS position (row r, slot s) must
+    // hold global chunk s ^ swz(r), so the swizzle is applied to the GLOBAL
+    // address each lane fetches from.  Rows outside the matrix (edge tiles) read
+    // as zero through the buffer descriptor's bounds check; that check covers
+    // the lane offset only, so the row part lives there and just the K offset
     // (always in range) goes into the scalar offset.
-    const int ld_row = tid >> 3, ld_chunk = tid & 7;
     const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<unsigned char*>(p.W), 0, (int)((size_t)p.N * p.K * ES), 0x00020000);
     const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<unsigned char*>(p.X), 0, (int)((((size_t)p.M - 1) * p.ldx + p.K) * ES), 0x00020000);
     const int w_rowb = p.K * ES, x_rowb = p.ldx * ES;
-    const int w_voff = ld_row * w_rowb + ld_chunk * 16;
-    const int x_voff = ld_row * x_rowb + ld_chunk * 16;
-    const int c0 = ld_chunk ^ ((ld_row ^ (ld_row >> 3)) & 7);
-    const int st_even = ld_row * 128 + (c0 << 4);
-    const int st_odd = ld_row * 128 + ((c0 ^ 4) << 4);
+    const int dr = lane >> 3;
+    const int dc = (lane & 7) ^ dr ^ wave;          // chunk fetched for even group index; odd: dc ^ 4
+    const int w_v0 = (n0 + 8 * wave + dr) * w_rowb + (dc << 4);
+    const int x_v0 = (m0 + 8 * wave + dr) * x_rowb + (dc << 4);
+    const int flip = ((dc ^ 4) - dc) << 4;          // +64 or -64 bytes
 
-    u32x4_t wreg[PASSES], xreg[PASSES];
-#define CUBERT_LOAD_GLOBAL(kt)                                                                         \
-    do {                                                                                               \
-        _Pragma("unroll") for (int i = 0; i < PASSES; ++i) {                                           \
-            wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(wres, w_voff + (n0 + i * 32) * w_rowb, (kt) * 128, 0); \
-            xreg[i] = __builtin_amdgcn_raw_buffer_load_b128(xres, x_voff + (m0 + i * 32) * x_rowb, (kt) * 128, 0); \
-        }                                                                                              \
-    } while (0)
-#define CUBERT_STORE_LDS(buf)                                                                          \
-    do {                                                                                               \
-        unsigned char* wt_ = smem + (buf) * 2 * TILE_BYTES;                                            \
-        unsigned char* xt_ = wt_ + TILE_BYTES;                                                         \
-        _Pragma("unroll") for (int i = 0; i < PASSES; ++i) {                                           \
-            const int off = i * 4096 + ((i & 1) ? st_odd : st_even);                                   \
-            *reinterpret_cast<u32x4_t*>(wt_ + off) = wreg[i];                                          \
-            *reinterpret_cast<u32x4_t*>(xt_ + off) = xreg[i];                                          \
-        }                                                                                              \
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+    const int KT = p.K / BK;
+    // A K step past the end (odd step counts run one phantom step) fetches from
+    // beyond the descriptor's range and therefore fills the tile with zeros.
+#define CUBERT_ISSUE_TILE(BUF, kt)                                                                          \
+    do {                                                                                                    \
+        const int oob = (kt) < KT ? 0 : 0x40000000;                                                         \
+        _Pragma("unroll") for (int i = 0; i < GROUPS; ++i) {                                                \
+            const int fl = (i & 1) ? flip : 0;                                                              \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(wres, (lds_ptr_t)((BUF) + (wave + 4 * i) * 1024), 16,  \
+                                                     (w_v0 + fl + i * 32 * w_rowb) | oob, (kt) * 128, 0, 0); \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (lds_ptr_t)((BUF) + TILE_BYTES + (wave + 4 * i) * 1024), \
+                                                     16, (x_v0 + fl + i * 32 * x_rowb) | oob, (kt) * 128, 0, 0); \
+        }                                                                                                   \
     } while (0)
 
     // ---- fragment read addressing ----
+    // Lane (row l32, group g) of 32x32 block i reads chunk 2*kk + g of tile row
+    // base + 32 i + l32, stored at slot (2*kk + g) ^ swz(row).  swz only depends
+    // on l32 and the parity of the block index, so the byte offset is
+    //   (off0 ^ ((i & 1) << 6) ^ (kk << 5)) + i * 4096
+    // with one lane-dependent base per operand.
     const int s0 = (l32 ^ (l32 >> 3)) & 7;
-    const int wrow0 = wn * (BT / 2) + l32;       // + 32*i
-    const int xrow0 = wm * (BT / 2) + l32;       // + 32*j
+    const int woff0 = (wn * (BT / 2) + l32) * 128 + ((g ^ s0 ^ (((wn * NB) & 1) << 2)) << 4);
+    const int xoff0 = TILE_BYTES + (wm * (BT / 2) + l32) * 128 + ((g ^ s0 ^ (((wm * NB) & 1) << 2)) << 4);
 
     f32x16_t acc[NB][NB];
 #pragma unroll
@@ -163,99 +140,55 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    const int KT = p.K / BK;
-    CUBERT_LOAD_GLOBAL(0);
-    CUBERT_STORE_LDS(0);
+#define CUBERT_LOAD_FRAGS(BUF, kk, WF, XF)                                                                  \
+    do {                                                                                                    \
+        _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                      \
+            WF[i] = *reinterpret_cast<const u32x4_t*>((BUF) + (wb ^ (((i & 1) << 6) ^ ((kk) << 5))) + i * 4096); \
+        _Pragma("unroll") for (int j = 0; j < NB; ++j)                                                      \
+            XF[j] = *reinterpret_cast<const u32x4_t*>((BUF) + (xb ^ (((j & 1) << 6) ^ ((kk) << 5))) + j * 4096); \
+    } while (0)
+
+    // One K step on buffer CUR while the loads for the next step fill NEXT.
+    // Fragments are double buffered in registers: the reads for k-step kk+1 are
+    // in flight while the MFMAs of k-step kk issue.  The empty asm keeps the
+    // compiler from hoisting (and then spilling) every per-k-step address.
+#define CUBERT_K_STEP(CUR, NEXT, kt)                                                                        \
+    do {                                                                                                    \
+        CUBERT_ISSUE_TILE(NEXT, (kt) + 1);                                                                  \
+        int wb = woff0, xb = xoff0;                                                                         \
+        asm volatile("" : "+v"(wb), "+v"(xb));                                                              \
+        u32x4_t wf[2][NB], xf[2][NB];                                                                       \
+        CUBERT_LOAD_FRAGS(CUR, 0, wf[0], xf[0]);                                                            \
+        _Pragma("unroll") for (int kk = 0; kk < 4; ++kk) {                                                  \
+            if (kk < 3) CUBERT_LOAD_FRAGS(CUR, kk + 1, wf[(kk + 1) & 1], xf[(kk + 1) & 1]);                 \
+            _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                  \
+                _Pragma("unroll") for (int j = 0; j < NB; ++j)                                              \
+                    mfma_chunk<ELT>(wf[kk & 1][i], xf[kk & 1][j], acc[i][j]);                               \
+        }                                                                                                   \
+        schedule_k_step<NB, MPC>();                                                                         \
+        __builtin_amdgcn_sched_barrier(0);  /* nothing moves across the end of the step */                  \
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): my share of NEXT has landed */                     \
+        __syncthreads();                                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                                  \
+    } while (0)
+
+    CUBERT_ISSUE_TILE(lds0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < KT) CUBERT_LOAD_GLOBAL(kt + 1);
-        const unsigned char* wt = smem + cur * 2 * TILE_BYTES;
-        const unsigned char* xt = wt + TILE_BYTES;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            u32x4_t wf[NB], xf[NB];
-#pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                const int row = wrow0 + 32 * i;
-                const int sw = s0 ^ ((((wn * (BT / 64)) + i) & 1) << 2);
-                wf[i] = *reinterpret_cast<const u32x4_t*>(wt + row * 128 + (((2 * kk + g) ^ sw) << 4));
-            }
-#pragma unroll
-            for (int j = 0; j < NB; ++j) {
-                const int row = xrow0 + 32 * j;
-                const int sw = s0 ^ ((((wm * (BT / 64)) + j) & 1) << 2);
-                xf[j] = *reinterpret_cast<const u32x4_t*>(xt + row * 128 + (((2 * kk + g) ^ sw) << 4));
-            }
-#pragma unroll
-            for (int i = 0; i < NB; ++i)
-#pragma unroll
-                for (int j = 0; j < NB; ++j) mfma_chunk<ELT>(wf[i], xf[j], acc[i][j]);
-        }
-        if (kt + 1 < KT) CUBERT_STORE_LDS(cur ^ 1);
-        __syncthreads();
+    for (int kt = 0; kt < KT; kt += 2) {
+        CUBERT_K_STEP(lds0, lds1, kt);
+        CUBERT_K_STEP(lds1, lds0, kt + 1);
     }
+#undef CUBERT_ISSUE_TILE
+#undef CUBERT_LOAD_FRAGS
+#undef CUBERT_K_STEP
 
-#undef CUBERT_LOAD_GLOBAL
-#undef CUBERT_STORE_LDS
-
-    // ---- epilogue: lane owns token (column) l32 and feature rows 8q+4g+e ----
-#pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int m = m0 + wm * (BT / 2) + 32 * j + l32;
-        if (m >= p.M) continue;
-        int bidx = 0, sidx = 0;
-        if constexpr (EPI == kEpiQKV) {
-            bidx = m / p.S;
-            sidx = m - bidx * p.S;
-        }
-#pragma unroll
-        for (int i = 0; i < NB; ++i) {
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int n = n0 + wn * (BT / 2) + 32 * i + 8 * qd + 4 * g;
-                if (n >= p.N) continue;
-                const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(p.bias + n);
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float t = acc[i][j][4 * qd + e] + b4[e];
-                    if constexpr (EPI == kEpiBiasGelu) t = gelu_erf(t);
-                    if constexpr (EPI == kEpiBiasTanh) t = tanhf(t);
-                    v[e] = t;
-                }
-                if constexpr (EPI == kEpiQKV) {
-                    const int which = n / p.hidden;
-                    const int hn = n - which * p.hidden;
-                    const int head = hn >> 6, dd = hn & 63;
-                    const size_t bh = (size_t)bidx * p.heads + head;
-                    if (which == 2) {
-                        const size_t base = (bh * 64 + dd) * p.Sp + sidx;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) store1<OUT>(p.vt, base + (size_t)e * p.Sp, v[e]);
-                    } else {
-                        store4<OUT>(which == 0 ? p.q : p.k, (bh * p.S + sidx) * 64 + dd, v);
-                    }
-                } else {
-                    store4<OUT>(p.Y, (size_t)m * p.N + n, v);
-                }
-            }
-        }
-    }
+    gemm_epilogue<OUT, EPI, NB>(p, acc, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g);
 }
 
 template <int ELT, int OUT, int EPI, int BT>
 bool launch_one(const GemmDev& d, hipStream_t stream) {
-    const size_t lds = (size_t)4 * BT * 128;     // two buffers x two operand tiles
-    auto kern = gemm_kernel<ELT, OUT, EPI, BT>;
-    static bool attr_done = false;               // per instantiation
-    if (!attr_done) {
-        CUBERT_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(d.tiles_n * d.tiles_m), dim3(256), lds, stream, d);
+    hipLaunchKernelGGL((gemm_kernel<ELT, OUT, EPI, BT>), dim3(d.tiles_n * d.tiles_m), dim3(256), 0, stream, d);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }
@@ -339,6 +272,9 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
     if (p.elt == kBF16) {
+        // 256 tile with an even number of K steps: the hand-scheduled kernel
+        if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled)
+            return launch_gemm_bf16_t256(d, out, p.epilogue, stream);
         return out == kBF16 ? launch_epi<kBF16, kBF16>(d, p.epilogue, bt, stream)
                             : launch_epi<kBF16, kF32>(d, p.epilogue, bt, stream);
     }

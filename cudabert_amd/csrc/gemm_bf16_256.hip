@@ -1,0 +1,106 @@
+// bf16 GEMM, 256x256 macro tile, hand-scheduled main loop (gfx950).
+//
+// Same operand roles (weights feed the MFMA "A" operand, activations "B") and
+// the same epilogue as the generic kernel in gemm.hip.  The whole K loop is one
+// inline-asm block (gemm_bf16_256_loop.inc, produced by gen_gemm_asm.py; the
+// pipeline, LDS map and register plan are described there) so that the order
+// of MFMAs, LDS fragment reads, global->LDS loads and waits is exactly the one
+// that keeps a single wave per SIMD busy.  Used when K is a multiple of 128
+// elements and the problem has enough tiles.
+#include "gemm_common.h"
+
+namespace cubert {
+namespace {
+
+using namespace gemm_detail;
+
+#define CUBERT_ACC_OPERANDS                                                                              \
+    [c00] "+a"(acc[0][0]), [c01] "+a"(acc[0][1]), [c02] "+a"(acc[0][2]), [c03] "+a"(acc[0][3]),         \
+    [c10] "+a"(acc[1][0]), [c11] "+a"(acc[1][1]), [c12] "+a"(acc[1][2]), [c13] "+a"(acc[1][3]),         \
+    [c20] "+a"(acc[2][0]), [c21] "+a"(acc[2][1]), [c22] "+a"(acc[2][2]), [c23] "+a"(acc[2][3]),         \
+    [c30] "+a"(acc[3][0]), [c31] "+a"(acc[3][1]), [c32] "+a"(acc[3][2]), [c33] "+a"(acc[3][3])
+
+#define CUBERT_V10(b) "v" #b "0", "v" #b "1", "v" #b "2", "v" #b "3", "v" #b "4", "v" #b "5", "v" #b "6", "v" #b "7", "v" #b "8", "v" #b "9"
+
+template <int OUT, int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
+    constexpr int BT = 256;
+    // Four stages of 32 KiB: W tile (256 rows x 64 B) then X tile.
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * 32768];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave >> 1, wm = wave & 1;
+    const int l32 = lane & 31, g = lane >> 5;
+
+    int tile_n, tile_m;
+    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, &tile_n, &tile_m);
+    const int n0 = tile_n * BT, m0 = tile_m * BT;
+
+    // Buffer descriptors as plain SGPR quads: base, base_hi (stride 0), num_records, flags.
+    // Rows outside the matrix read as zero (bounds check on the lane offset).
+    const unsigned long long wa = reinterpret_cast<unsigned long long>(p.W);
+    const unsigned long long xa = reinterpret_cast<unsigned long long>(p.X);
+    const u32x4_t wres = {(unsigned)wa, (unsigned)(wa >> 32) & 0xffffu, (unsigned)((size_t)p.N * p.K * 2), 0x00020000u};
+    const u32x4_t xres = {(unsigned)xa, (unsigned)(xa >> 32) & 0xffffu,
+                          (unsigned)((((size_t)p.M - 1) * p.ldx + p.K) * 2), 0x00020000u};
+    const int w_rowb = p.K * 2, x_rowb = p.ldx * 2;
+    // global->LDS: one load moves 16 rows; lane fetches row 16*group + lane/4 and the chunk
+    // that belongs into its LDS slot lane%4 (slot = chunk ^ swz(row)).  Wave w moves the
+    // groups w, w+4, w+8, w+12, for which swz only depends on the lane and the parity of w.
+    const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
+    const int w_v0 = (n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4);
+    const int x_v0 = (m0 + 16 * wave + (lane >> 2)) * x_rowb + (dc << 4);
+    const int w64 = 64 * w_rowb, x64 = 64 * x_rowb;
+    // fragment reads: chunk g of my row in the W / X tile of stage 0, k-phase 0
+    const int lds_base = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
+    const int wb = lds_base + (wn * 128 + l32) * 64 + ((g ^ sw) << 4);
+    const int xb = lds_base + 16384 + (wm * 128 + l32) * 64 + ((g ^ sw) << 4);
+    const int m0b = lds_base + wave * 1024;
+    const int ht = p.K / 32;          // half-steps; a multiple of 4
+
+    f32x16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    asm volatile(
+#include "gemm_bf16_256_loop.inc"
+        : CUBERT_ACC_OPERANDS
+        : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
+          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b)
+        : "memory", "scc", "s92", "s93", "s94", "s95", "s96", "s97", "v176", "v177", "v178", "v179",
+          CUBERT_V10(18), CUBERT_V10(19), CUBERT_V10(20), CUBERT_V10(21), CUBERT_V10(22), CUBERT_V10(23),
+          CUBERT_V10(24), "v250", "v251", "v252", "v253", "v254", "v255");
+
+    gemm_epilogue<OUT, EPI, 4>(p, acc, n0 + wn * 128, m0 + wm * 128, l32, g);
+}
+
+template <int OUT>
+bool launch_epi(const GemmDev& d, int epi, hipStream_t stream) {
+    const dim3 grid(d.tiles_n * d.tiles_m), block(256);
+    switch (epi) {
+        case kEpiBias: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBias>), grid, block, 0, stream, d); break;
+        case kEpiBiasGelu: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasGelu>), grid, block, 0, stream, d); break;
+        case kEpiBiasTanh: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasTanh>), grid, block, 0, stream, d); break;
+        case kEpiQKV: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiQKV>), grid, block, 0, stream, d); break;
+        default: set_error("gemm: unknown epilogue"); return false;
+    }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+}  // namespace
+
+// d.tiles_n / d.tiles_m must have been computed for a 256 tile and d.K % 128 == 0.
+bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream) {
+    if (d.K % 128 != 0 || d.K < 128) { set_error("gemm: the 256 tile needs K to be a multiple of 128"); return false; }
+    return out_elt == kBF16 ? launch_epi<kBF16>(d, epilogue, stream) : launch_epi<kF32>(d, epilogue, stream);
+}
+
+}  // namespace cubert

@@ -1,0 +1,142 @@
+// Pieces shared by the GEMM kernels: the launch descriptor, small device
+// helpers, the workgroup -> tile mapping and the epilogue.
+#pragma once
+#include "kernels.h"
+
+namespace cubert {
+namespace gemm_detail {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+
+struct GemmDev {
+    const unsigned char* X;
+    const unsigned char* W;
+    const float* bias;
+    unsigned char* Y;
+    unsigned char* q;
+    unsigned char* k;
+    unsigned char* vt;
+    int M, N, K, ldx;
+    int S, Sp, heads, hidden;
+    int tiles_n, tiles_m;
+};
+
+__device__ __forceinline__ float gelu_erf(float x) {
+    return x * 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+// GELU with erf from Abramowitz & Stegun 7.1.26 (|error| < 1.5e-7, far below
+// bf16 resolution); used when the result is stored as bf16.
+__device__ __forceinline__ float gelu_fast(float x) {
+    const float z = fabsf(x) * 0.70710678118654752440f;
+    const float t = __frcp_rn(1.0f + 0.3275911f * z);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    const float erf_abs = 1.0f - poly * __expf(-z * z);
+    return 0.5f * x * (1.0f + copysignf(erf_abs, x));
+}
+
+template <int ELT>
+__device__ __forceinline__ void mfma_chunk(const u32x4_t& a, const u32x4_t& b, f32x16_t& acc) {
+    if constexpr (ELT == kBF16) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                      __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+    } else {
+        const f32x4_t fa = __builtin_bit_cast(f32x4_t, a);
+        const f32x4_t fb = __builtin_bit_cast(f32x4_t, b);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1], fb[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2], fb[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[3], fb[3], acc, 0, 0, 0);
+    }
+}
+
+template <int OUT>
+__device__ __forceinline__ void store4(unsigned char* base, size_t elem_index, const float v[4]) {
+    if constexpr (OUT == kBF16) {
+        bf16x4_t o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+        *reinterpret_cast<bf16x4_t*>(base + elem_index * 2) = o;
+    } else {
+        f32x4_t o = {v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<f32x4_t*>(base + elem_index * 4) = o;
+    }
+}
+
+template <int OUT>
+__device__ __forceinline__ void store1(unsigned char* base, size_t elem_index, float v) {
+    if constexpr (OUT == kBF16) {
+        *reinterpret_cast<__bf16*>(base + elem_index * 2) = (__bf16)v;
+    } else {
+        *reinterpret_cast<float*>(base + elem_index * 4) = v;
+    }
+}
+
+// Workgroup id -> (tile_n, tile_m).  Hardware hands consecutive workgroup ids
+// to the eight XCDs round-robin; the remap gives every XCD one contiguous run
+// of the tile sequence so tiles sharing operand rows share an L2.
+__device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int* tn, int* tm) {
+    const int xcd = pid & 7, idx = pid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    const int start = xcd * base + (xcd < rem ? xcd : rem);
+    const int t = start + idx;
+    *tm = t / tiles_n;
+    *tn = t - *tm * tiles_n;
+}
+
+
+// Epilogue.  In the 32x32 accumulator layout lane (l32 = lane % 32, g = lane / 32)
+// owns token column l32 of block j and, per accumulator quad qd, the four
+// consecutive feature rows 8 qd + 4 g + {0..3} of block i.  n_base / m_base are
+// the first feature / token of this wave's quadrant.
+template <int OUT, int EPI, int NB>
+__device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NB][NB], int n_base, int m_base,
+                                              int l32, int g) {
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int m = m_base + 32 * j + l32;
+        if (m >= p.M) continue;
+        int bidx = 0, sidx = 0;
+        if constexpr (EPI == kEpiQKV) {
+            bidx = m / p.S;
+            sidx = m - bidx * p.S;
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int n = n_base + 32 * i + 8 * qd + 4 * g;
+                if (n >= p.N) continue;
+                const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(p.bias + n);
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float t = acc[i][j][4 * qd + e] + b4[e];
+                    if constexpr (EPI == kEpiBiasGelu) t = (OUT == kBF16) ? gelu_fast(t) : gelu_erf(t);
+                    if constexpr (EPI == kEpiBiasTanh) t = tanhf(t);
+                    v[e] = t;
+                }
+                if constexpr (EPI == kEpiQKV) {
+                    const int which = n / p.hidden;
+                    const int hn = n - which * p.hidden;
+                    const int head = hn >> 6, dd = hn & 63;
+                    const size_t bh = (size_t)bidx * p.heads + head;
+                    if (which == 2) {
+                        const size_t base = (bh * 64 + dd) * p.Sp + sidx;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) store1<OUT>(p.vt, base + (size_t)e * p.Sp, v[e]);
+                    } else {
+                        store4<OUT>(which == 0 ? p.q : p.k, (bh * p.S + sidx) * 64 + dd, v);
+                    }
+                } else {
+                    store4<OUT>(p.Y, (size_t)m * p.N + n, v);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace gemm_detail
+}  // namespace cubert

@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Generates gemm_bf16_256_loop.inc: the hand-scheduled main loop (gfx950 ISA,
+as one inline-asm string) of the 256x256 bf16 GEMM macro tile.
+
+    python gen_gemm_asm.py > gemm_bf16_256_loop.inc
+
+Why hand-scheduled: with 256 accumulator registers per lane a SIMD holds one
+wave, so nothing but instruction order hides LDS and memory latency.
+
+Pipeline.  K is consumed in half-steps of 32 bf16 (64 bytes per tile row).  LDS
+holds four stages of 32 KiB (W tile 256 rows x 64 B, then X tile); the tile of
+half-step h lives in stage h % 4.  During half-step h a wave
+  * issues 32 MFMAs (32x32x16): k-phase 0 on fragment set A, k-phase 1 on set B,
+  * reads the k-phase-1 fragments of tile h (into B) behind the first MFMAs of
+    phase 0 and the k-phase-0 fragments of tile h+1 (into A) behind the first
+    MFMAs of phase 1, so no fragment read is ever waited for right after issue,
+  * issues its 8 global->LDS loads of tile h+3 (three half-steps ahead, which
+    keeps a steady stream of requests in flight instead of one burst per step),
+  * ends with "s_waitcnt vmcnt(8)" -- everything but the 8 loads just issued,
+    i.e. tile h+2, has landed -- and one s_barrier.
+The barrier at the end of half-step h-1 therefore guarantees tile h+1, which is
+what lets half-step h prefetch tile h+1's fragments before its own barrier.
+
+Register plan (per lane):
+  a[0:255]    accumulators: 4x4 blocks of 32x32 (inline-asm "+a" operands)
+  v[192:207]  W fragments, set A (block i at 192+4i)   v[208:223]  X fragments, set A
+  v[224:239]  W fragments, set B                       v[240:255]  X fragments, set B
+  v[176:179]  LDS byte addresses of my fragment row in stage 0: W k-phase 0, W k-phase 1,
+              X k-phase 0, X k-phase 1                 v[180:183]  the same + 65536 (stages 2, 3)
+  v[184:187]  global lane offsets of my 4 W row groups v[188:191]  same for X
+  s96 K byte offset of the tile being fetched, s97 loop counter,
+  s92..s95    M0 base of stage 0..3 (stage base + wave * 1024)
+
+LDS swizzle: a tile row is 64 bytes = four 16-byte chunks; chunk c of row r sits
+in slot c ^ (((r >> 1) ^ (r >> 3)) & 3), which spreads the fragment reads of any
+8 or 16 consecutive rows over all banks.  One buffer_load_dwordx4 ... lds moves
+16 rows (64 lanes x 16 B) to M0 + 16 * lane; the swizzle is applied on the
+global side (which chunk a lane fetches).
+"""
+import os
+
+# Ablation switches for timing experiments only (they break the result).
+ABL = set(os.environ.get("CUBERT_GEMM_ABLATE", "").split(","))
+
+WA, XA, WB, XB = 192, 208, 224, 240
+ADDR = 176            # + 4 * bank + {0: W kk0, 1: W kk1, 2: X kk0, 3: X kk1}
+W_VOFF, X_VOFF = 184, 188
+NSTAGE = 4
+
+
+def vreg4(base):
+    return "v[%d:%d]" % (base, base + 3)
+
+
+class Emitter:
+    def __init__(self):
+        self.lines = []
+        self.issued = 0            # LDS reads issued so far (monotonic)
+        self.index = {}            # fragment register base -> issue index of its latest read
+        self.guaranteed = None     # an upper bound on outstanding LDS reads already waited for
+
+    def emit(self, text):
+        if "nodma" in ABL and text.startswith("buffer_load_dwordx4"):
+            return
+        if "noread" in ABL and text.startswith("ds_read"):
+            return
+        if "nomfma" in ABL and text.startswith("v_mfma"):
+            return
+        self.lines.append(text)
+
+    def read(self, dst, addr_reg, offset):
+        assert 0 <= offset < 65536
+        self.emit("ds_read_b128 %s, v%d offset:%d" % (vreg4(dst), addr_reg, offset))
+        self.index[dst] = self.issued
+        self.issued += 1
+        if self.guaranteed is not None:
+            self.guaranteed += 1
+
+    def need(self, *regs):
+        """Weakest s_waitcnt that guarantees the reads into `regs` have returned
+        (LDS reads return in order)."""
+        newest = max(self.index[r] for r in regs)
+        allowed = self.issued - 1 - newest
+        if self.guaranteed is None or allowed < self.guaranteed:
+            self.emit("s_waitcnt lgkmcnt(%d)" % min(allowed, 15))
+            self.guaranteed = allowed
+
+    def forget_bound(self):
+        self.guaranteed = None
+
+
+READ_ORDER = [("w", 0), ("x", 0), ("x", 1), ("x", 2), ("x", 3), ("w", 1), ("w", 2), ("w", 3)]
+
+
+def frag_reads(stage, kk, wset, xset):
+    bank, half = stage >> 1, stage & 1
+    out = []
+    for kind, b in READ_ORDER:
+        if kind == "w":
+            out.append((wset + 4 * b, ADDR + 4 * bank + kk, half * 32768 + b * 2048))
+        else:
+            out.append((xset + 4 * b, ADDR + 4 * bank + 2 + kk, half * 32768 + b * 2048))
+    return out
+
+
+def dma_instrs(stage):
+    """The eight global->LDS loads of one tile into `stage`: (M0 update, load)."""
+    out = []
+    for k in range(8):
+        m0 = ("s_mov_b32 m0, s%d" % (92 + stage)) if k == 0 else "s_add_u32 m0, m0, 0x1000"
+        if k < 4:
+            ld = "buffer_load_dwordx4 v%d, %%[wres], s96 offen lds" % (W_VOFF + k)
+        else:
+            ld = "buffer_load_dwordx4 v%d, %%[xres], s96 offen lds" % (X_VOFF + k - 4)
+        out.append((m0, ld))
+    return out
+
+
+def half_step(e, stage, dma, prefetch_next, vmcnt, barrier):
+    """One half-step on `stage`.  On entry the 8 reads of set A (k-phase 0 of this
+    tile) have been issued, in READ_ORDER, as the latest 8 LDS reads."""
+    e.emit("; ---- half-step on stage %d%s" % (stage, ", fetch into stage %d" % ((stage + 3) % NSTAGE) if dma else ""))
+    dmas = dma_instrs((stage + 3) % NSTAGE) if dma else []
+    for kk in range(2):
+        wset, xset = (WA, XA) if kk == 0 else (WB, XB)
+        if kk == 0:
+            pending = frag_reads(stage, 1, WB, XB)
+        else:
+            pending = frag_reads((stage + 1) % NSTAGE, 0, WA, XA) if prefetch_next else []
+        m = 0
+        for i in range(4):
+            for j in range(4):
+                e.need(wset + 4 * i, xset + 4 * j)
+                d = m // 2 if (kk == 0 and dmas and m % 2 == 0) else None
+                if d is not None:
+                    e.emit(dmas[d][0])      # M0 update in front of the MFMA: the MFMA is the
+                e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %   # wait state before M0 is used
+                       (i, j, vreg4(wset + 4 * i), vreg4(xset + 4 * j), i, j))
+                if d is not None:
+                    e.emit(dmas[d][1])
+                # The destination set of these reads was last used by MFMAs of the
+                # previous k-phase, all of which have issued.
+                if m < len(pending):
+                    e.read(*pending[m])
+                m += 1
+    if vmcnt is not None:
+        e.emit("s_waitcnt vmcnt(%d)" % vmcnt)
+    if barrier:
+        e.emit("s_barrier")
+
+
+def main():
+    e = Emitter()
+    e.emit("; ======== setup ========")
+    e.emit("v_mov_b32 v%d, %%[wb]" % (ADDR + 0))
+    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (ADDR + 1))
+    e.emit("v_mov_b32 v%d, %%[xb]" % (ADDR + 2))
+    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (ADDR + 3))
+    for r in range(4):
+        e.emit("v_add_u32 v%d, 0x10000, v%d" % (ADDR + 4 + r, ADDR + r))
+    e.emit("v_mov_b32 v%d, %%[wv0]" % W_VOFF)
+    e.emit("v_mov_b32 v%d, %%[xv0]" % X_VOFF)
+    for i in range(1, 4):
+        e.emit("v_add_u32 v%d, %%[w64], v%d" % (W_VOFF + i, W_VOFF + i - 1))
+        e.emit("v_add_u32 v%d, %%[x64], v%d" % (X_VOFF + i, X_VOFF + i - 1))
+    e.emit("s_mov_b32 s92, %[m0b]")
+    for s in range(1, NSTAGE):
+        e.emit("s_add_u32 s%d, s%d, 0x8000" % (92 + s, 92 + s - 1))
+    e.emit("; ======== prologue: tiles 0, 1, 2 -> stages 0, 1, 2 ========")
+    e.emit("s_mov_b32 s96, 0")
+    for t in range(3):
+        for m0, ld in dma_instrs(t):
+            e.emit(m0)
+            e.emit("s_nop 0")
+            e.emit(ld)
+        if t < 2:
+            e.emit("s_add_u32 s96, s96, 64")
+    e.emit("s_waitcnt vmcnt(8)")          # tiles 0 and 1 have landed
+    e.emit("s_barrier")
+    for r in frag_reads(0, 0, WA, XA):
+        e.read(*r)
+    e.emit("s_mov_b32 s97, 4")
+    e.emit("s_cmp_ge_u32 s97, %[ht]")
+    e.emit("s_cbranch_scc1 L_tail_%=")
+    e.emit("L_loop_%=:")
+    for s in range(NSTAGE):
+        e.emit("s_add_u32 s96, s96, 64")
+        half_step(e, s, dma=True, prefetch_next=True, vmcnt=8, barrier=True)
+    e.forget_bound()                       # the loop head is reached from two places
+    e.emit("s_add_u32 s97, s97, 4")
+    e.emit("s_cmp_lt_u32 s97, %[ht]")
+    e.emit("s_cbranch_scc1 L_loop_%=")
+    e.emit("L_tail_%=:")
+    e.forget_bound()
+    e.emit("s_add_u32 s96, s96, 64")
+    half_step(e, 0, dma=True, prefetch_next=True, vmcnt=8, barrier=True)      # fetches the last tile
+    half_step(e, 1, dma=False, prefetch_next=True, vmcnt=0, barrier=True)
+    half_step(e, 2, dma=False, prefetch_next=True, vmcnt=None, barrier=False)
+    half_step(e, 3, dma=False, prefetch_next=False, vmcnt=None, barrier=False)
+    print("// Generated by gen_gemm_asm.py -- do not edit.")
+    for ln in e.lines:
+        print('"%s\\n"' % ln)
+
+
+if __name__ == "__main__":
+    main()

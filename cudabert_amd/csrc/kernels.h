@@ -42,6 +42,7 @@ struct GemmParams {
     void* vt = nullptr;
     int S = 0, Sp = 0, heads = 0;
     int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile)
+    bool compiler_scheduled = false;   // 256 tile: use the generic kernel, not the hand-scheduled one
 };
 bool launch_gemm(const GemmParams& p, hipStream_t stream);
 
