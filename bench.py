@@ -131,17 +131,23 @@ def main():
                            "frac_mfma_peak": round(gemm_flops / gemm_ms / 1e9 / PEAK_TFLOPS[args.precision], 4)}
 
     # ---- roofline of the dominant kernel: the FFN-in GEMM (bias+GELU epilogue) ----
+    # Same launch as in the model: in bf16 mode all three matrices are in the packed
+    # operand layout (their contents are random, only the layout matters for timing).
     tdt = torch.bfloat16 if prec == pybert.BF16 else torch.float32
-    X = (torch.randn((N, H), device="cuda") * 1.0).to(tdt)
-    Wt = (torch.randn((I, H), device="cuda") * 0.02).to(tdt)
+    packed = prec == pybert.BF16
+    rows_x = (N + 255) // 256 * 256 if packed else N
+    rows_w = (I + 255) // 256 * 256 if packed else I
+    X = (torch.randn((rows_x, H), device="cuda") * 1.0).to(tdt)
+    Wt = (torch.randn((rows_w, H), device="cuda") * 0.02).to(tdt)
     bias = torch.zeros(I, device="cuda")
-    Y = torch.empty((N, I), dtype=tdt, device="cuda")
+    Y = torch.empty((rows_x, I), dtype=tdt, device="cuda")
     st = torch.cuda.current_stream()
     out_elt = prec
+    gflags = (pybert.X_PACKED | pybert.W_PACKED | pybert.Y_PACKED) if packed else 0
 
     def ffn_in():
         pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H, prec,
-                                        out_elt, 1, 0, st.cuda_stream))
+                                        out_elt, 1, 0, gflags, st.cuda_stream))
     for _ in range(3):
         ffn_in()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -30,7 +30,7 @@ template <int ELT>
 __global__ __launch_bounds__(256) void attention_kernel(
     const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
     const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
-    unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale) {
+    unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale, int ctx_packed) {
     constexpr int ES = (ELT == kBF16) ? 2 : 4;
     constexpr int ROWB = 64 * ES;            // bytes per Q/K row
     constexpr int KK = ROWB / 32;            // MFMA k-steps over the head dim (4 bf16 / 8 f32)
@@ -159,7 +159,10 @@ __global__ __launch_bounds__(256) void attention_kernel(
             if constexpr (ELT == kBF16) {
                 bf16x4_t w = {(__bf16)(o[db][4 * j] * inv), (__bf16)(o[db][4 * j + 1] * inv),
                               (__bf16)(o[db][4 * j + 2] * inv), (__bf16)(o[db][4 * j + 3] * inv)};
-                *reinterpret_cast<bf16x4_t*>(orow + d * 2) = w;
+                if (ctx_packed)
+                    *reinterpret_cast<bf16x4_t*>(ctx + packed_offset(b * S + qi, (h * 64 + d) * 2, (int)hidden * 2 / 64)) = w;
+                else
+                    *reinterpret_cast<bf16x4_t*>(orow + d * 2) = w;
             } else {
                 f32x4_t w = {o[db][4 * j] * inv, o[db][4 * j + 1] * inv, o[db][4 * j + 2] * inv,
                              o[db][4 * j + 3] * inv};
@@ -171,7 +174,9 @@ __global__ __launch_bounds__(256) void attention_kernel(
 }  // namespace
 
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
-                      int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream) {
+                      bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream) {
+    if (ctx_packed && elt != kBF16) { set_error("attention: only a bf16 context can be packed"); return false; }
+    const int cp = ctx_packed ? 1 : 0;
     if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
     if (B <= 0 || heads <= 0 || S <= 0) { set_error("attention: empty problem"); return false; }
     if (Sp % 32 != 0 || Sp < S || Sp - S >= 32) {
@@ -191,9 +196,9 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
     const unsigned char* vc = static_cast<const unsigned char*>(vt);
     unsigned char* cc = static_cast<unsigned char*>(ctx);
     if (elt == kBF16)
-        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale);
+        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp);
     else
-        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale);
+        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }

@@ -235,51 +235,72 @@ void test(int batchsize, int seq_length, int nIter, bool large, int num_gpu) {
 
 // ------------------------------------------------------------ single ops ---
 
+namespace {
+void apply_gemm_flags(cubert::GemmParams* p, int flags) {
+    p->x_packed = (flags & CUBERT_X_PACKED) != 0;
+    p->w_packed = (flags & CUBERT_W_PACKED) != 0;
+    p->y_packed = (flags & CUBERT_Y_PACKED) != 0;
+    p->compiler_scheduled = (flags & CUBERT_COMPILER_SCHEDULED) != 0;
+}
+}  // namespace
+
 int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int M, int N, int K, int ldx, int elt,
-                   int out_elt, int epilogue, int tile, void* stream) {
+                   int out_elt, int epilogue, int tile, int flags, void* stream) {
     cubert::set_error("");
     if (epilogue < 0 || epilogue > 2) { cubert::set_error("cubert_op_gemm: epilogue must be 0, 1 or 2"); return 1; }
     cubert::GemmParams p;
     p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.elt = elt;
     p.out_elt = out_elt; p.epilogue = epilogue; p.tile = tile;
-    if (tile == 257) { p.tile = 256; p.compiler_scheduled = true; }   // 256 tile, generic (compiler-scheduled) kernel
+    apply_gemm_flags(&p, flags);
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
 int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q, void* k, void* vt, int B, int S,
-                       int heads, int elt, int tile, void* stream) {
+                       int heads, int elt, int tile, int flags, void* stream) {
     cubert::set_error("");
     if (B <= 0 || S <= 0 || heads <= 0) { cubert::set_error("cubert_op_gemm_qkv: bad shape"); return 1; }
     cubert::GemmParams p;
     p.X = X; p.W = W; p.bias = bias; p.M = B * S; p.N = 3 * heads * 64; p.K = heads * 64; p.ldx = heads * 64;
     p.elt = elt; p.epilogue = cubert::kEpiQKV; p.q = q; p.k = k; p.vt = vt; p.S = S; p.Sp = cubert::round_up(S, 32);
     p.heads = heads; p.tile = tile;
-    if (tile == 257) { p.tile = 256; p.compiler_scheduled = true; }
+    apply_gemm_flags(&p, flags);
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
+size_t cubert_packed_bytes(size_t rows, size_t row_bytes) { return cubert::packed_bytes(rows, row_bytes); }
+size_t cubert_packed_offset(int row, int kbyte, int row_bytes) { return cubert::packed_offset(row, kbyte, row_bytes / 64); }
+
 int cubert_op_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx, int B,
-                        int heads, int S, float scale, int elt, void* stream) {
+                        int heads, int S, float scale, int elt, int flags, void* stream) {
     cubert::set_error("");
-    return cubert::launch_attention(q, k, vt, maskadd, ctx, B, heads, S, cubert::round_up(S > 0 ? S : 1, 32), scale,
-                                    elt, static_cast<hipStream_t>(stream)) ? 0 : 1;
+    return cubert::launch_attention(q, k, vt, maskadd, ctx, (flags & CUBERT_Y_PACKED) != 0, B, heads, S,
+                                    cubert::round_up(S > 0 ? S : 1, 32), scale, elt,
+                                    static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
 int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta, void* xb,
-                            int rows, int hidden, void* stream) {
+                            int rows, int hidden, int flags, void* stream) {
     cubert::set_error("");
-    return cubert::launch_add_layernorm(x, y, y_elt, gamma, beta, static_cast<cubert::bf16_t*>(xb), rows, hidden,
+    return cubert::launch_add_layernorm(x, y, y_elt, gamma, beta, static_cast<cubert::bf16_t*>(xb),
+                                        (flags & CUBERT_Y_PACKED) != 0, rows, hidden,
                                         static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
 int cubert_op_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word, const float* pos,
                               const float* type, const float* gamma, const float* beta, float* x, void* xb,
-                              float* maskadd, int B, int S, int hidden, int vocab, int type_vocab, void* stream) {
+                              float* maskadd, int B, int S, int hidden, int vocab, int type_vocab, int flags,
+                              void* stream) {
     cubert::set_error("");
     return cubert::launch_embed_layernorm(ids, seg, mask, word, pos, type, gamma, beta, x,
-                                          static_cast<cubert::bf16_t*>(xb), maskadd, B, S,
+                                          static_cast<cubert::bf16_t*>(xb), (flags & CUBERT_Y_PACKED) != 0, maskadd, B, S,
                                           cubert::round_up(S > 0 ? S : 1, 32), hidden, vocab, type_vocab,
                                           static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+int cubert_op_pooler(const float* x, const void* W, const float* bias, float* pooled, int B, int S, int hidden,
+                     int w_elt, void* stream) {
+    cubert::set_error("");
+    return cubert::launch_pooler(x, W, w_elt, bias, pooled, B, S, hidden, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
 int cubert_op_mask_softmax(void* scores, int elt, const int* mask, int B, int rows_per_batch, int S, float scale,

@@ -92,11 +92,13 @@ bool Model::init(const ModelOptions& opt_in) {
     Arena wa;
     const size_t o_word = wa.take((size_t)D.vocab * H * 4), o_pos = wa.take((size_t)D.max_pos * H * 4),
                  o_type = wa.take((size_t)D.type_vocab * H * 4), o_eg = wa.take(H * 4), o_eb = wa.take(H * 4);
+    auto wbytes = [&](size_t rows, size_t k) { return elt == kBF16 ? packed_bytes(rows, k * 2) : rows * k * es; };
     struct LayerOff { size_t w_qkv, w_ao, w_in, w_out, b_qkv, b_ao, b_in, b_out, g1, be1, g2, be2; };
     std::vector<LayerOff> lo(D.layers);
     for (auto& l : lo) {
-        l.w_qkv = wa.take(3 * H * H * es); l.w_ao = wa.take(H * H * es);
-        l.w_in = wa.take(I * H * es); l.w_out = wa.take(H * I * es);
+        // packed operands (bf16 mode) pad their rows to a multiple of 256
+        l.w_qkv = wa.take(wbytes(3 * H, H)); l.w_ao = wa.take(wbytes(H, H));
+        l.w_in = wa.take(wbytes(I, H)); l.w_out = wa.take(wbytes(H, I));
         l.b_qkv = wa.take(3 * H * 4); l.b_ao = wa.take(H * 4); l.b_in = wa.take(I * 4); l.b_out = wa.take(H * 4);
         l.g1 = wa.take(H * 4); l.be1 = wa.take(H * 4); l.g2 = wa.take(H * 4); l.be2 = wa.take(H * 4);
     }
@@ -114,10 +116,18 @@ bool Model::init(const ModelOptions& opt_in) {
     };
     // [in, out] float32 on disk -> [out, in] operand type on device
     float* stage = reinterpret_cast<float*>(wblock_ + o_stage);
-    auto up_t = [&](size_t off, const NpyArray* a) -> bool {
+    // bf16 mode keeps GEMM operands in the packed layout (common.h); the pooler
+    // weight stays row-major (its kernel is a plain dot product).
+    const bool packed = elt == kBF16;
+    bool pack_this = true;
+    // `row0`: first output row of this tensor inside the destination matrix (the
+    // Q, K and V kernels are stacked into one [3H, H] operand).
+    auto up_t = [&](size_t off, const NpyArray* a, int row0 = 0) -> bool {
         const int K = (int)a->shape[0], N = (int)a->shape[1];
         CUBERT_HIP_OK(hipMemcpyAsync(stage, a->data.data(), a->data.size() * 4, hipMemcpyHostToDevice, stream_));
-        if (!launch_transpose_convert(stage, wblock_ + off, K, N, elt, stream_)) return false;
+        const bool pk = packed && pack_this;
+        unsigned char* dst = wblock_ + off + (pk ? 0 : (size_t)row0 * K * es);
+        if (!launch_transpose_convert(stage, dst, K, N, elt, pk, pk ? row0 : 0, stream_)) return false;
         CUBERT_HIP_OK(hipStreamSynchronize(stream_));      // the staging buffer is reused
         return true;
     };
@@ -134,7 +144,7 @@ bool Model::init(const ModelOptions& opt_in) {
         const LayerOff& l = lo[i];
         // Q, K, V stacked along the output axis: rows [0,H) query, [H,2H) key, [2H,3H) value
         // (the reference concatenates them too, cuda_bert/ops/linear.cu:60-88).
-        if (!up_t(l.w_qkv, T.q_k) || !up_t(l.w_qkv + H * H * es, T.k_k) || !up_t(l.w_qkv + 2 * H * H * es, T.v_k) ||
+        if (!up_t(l.w_qkv, T.q_k, 0) || !up_t(l.w_qkv, T.k_k, (int)H) || !up_t(l.w_qkv, T.v_k, 2 * (int)H) ||
             !up_t(l.w_ao, T.ao_k) || !up_t(l.w_in, T.in_k) || !up_t(l.w_out, T.out_k))
             return false;
         if (!up(l.b_qkv, T.q_b) || !up(l.b_qkv + H * 4, T.k_b) || !up(l.b_qkv + 2 * H * 4, T.v_b) ||
@@ -148,6 +158,7 @@ bool Model::init(const ModelOptions& opt_in) {
         L.g1 = reinterpret_cast<float*>(wblock_ + l.g1); L.be1 = reinterpret_cast<float*>(wblock_ + l.be1);
         L.g2 = reinterpret_cast<float*>(wblock_ + l.g2); L.be2 = reinterpret_cast<float*>(wblock_ + l.be2);
     }
+    pack_this = false;
     if (!up_t(o_wp, wd.pool_k) || !up(o_bp, wd.pool_b)) return false;
     w_pool_ = wblock_ + o_wp;
     b_pool_ = reinterpret_cast<float*>(wblock_ + o_bp);
@@ -159,7 +170,7 @@ bool Model::init(const ModelOptions& opt_in) {
 
     // ---- activation block: one allocation, addresses fixed for the model's life ----
     // B <= 1024 and every sequence is padded by < 32 key columns in vt/maskadd.
-    const size_t N = (size_t)cap_tokens_;
+    const size_t N = ((size_t)cap_tokens_ + 255) / 256 * 256;     // packed operands pad rows to 256
     const size_t Npad = N + 32 * 1024;
     Arena aa;
     const size_t o_x32 = aa.take(N * H * 4);
@@ -288,8 +299,9 @@ bool Model::enqueue(int B, int S, bool has_mask) {
     const float scale = 1.0f / std::sqrt(64.0f);
 
     if (!mark(kPhEmbed)) return false;
-    if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32_, xb_, maskadd_, B, S, Sp, H,
-                                D.vocab, D.type_vocab, stream_))
+    const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
+    if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32_, xb_, pk, maskadd_, B, S, Sp,
+                                H, D.vocab, D.type_vocab, stream_))
         return false;
     for (int i = 0; i < D.layers; ++i) {
         const LayerDev& L = layers_[i];
@@ -298,34 +310,32 @@ bool Model::enqueue(int B, int S, bool has_mask) {
         // QKV projection, scattered per head (V transposed)
         g.X = xin; g.ldx = H; g.W = L.w_qkv; g.bias = L.b_qkv; g.M = N; g.N = 3 * H; g.K = H;
         g.epilogue = kEpiQKV; g.q = q_; g.k = k_; g.vt = vt_; g.S = S; g.Sp = Sp; g.heads = D.heads;
+        g.x_packed = g.w_packed = pk;
         if (!mark(kPhQKV) || !launch_gemm(g, stream_)) return false;
         if (!mark(kPhAttention)) return false;
-        if (!launch_attention(q_, k_, vt_, maskadd_, ctx_, B, D.heads, S, Sp, scale, elt, stream_)) return false;
+        if (!launch_attention(q_, k_, vt_, maskadd_, ctx_, pk, B, D.heads, S, Sp, scale, elt, stream_)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx_; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32_;
-        g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias;
+        g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
         if (!mark(kPhAttnOut) || !launch_gemm(g, stream_)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32_, y32_, kF32, L.g1, L.be1, xb_, N, H, stream_)) return false;
+        if (!launch_add_layernorm(x32_, y32_, kF32, L.g1, L.be1, xb_, pk, N, H, stream_)) return false;
         // feed-forward
         g = GemmParams();
         g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h_;
-        g.M = N; g.N = I; g.K = H; g.epilogue = kEpiBiasGelu;
+        g.M = N; g.N = I; g.K = H; g.epilogue = kEpiBiasGelu; g.x_packed = g.w_packed = g.y_packed = pk;
         if (!mark(kPhFFNIn) || !launch_gemm(g, stream_)) return false;
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = h_; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32_;
-        g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias;
+        g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
         if (!mark(kPhFFNOut) || !launch_gemm(g, stream_)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32_, y32_, kF32, L.g2, L.be2, xb_, N, H, stream_)) return false;
+        if (!launch_add_layernorm(x32_, y32_, kF32, L.g2, L.be2, xb_, pk, N, H, stream_)) return false;
     }
-    // pooler: tanh(dense(first token)); the first-token gather is the row stride S*H
-    GemmParams g;
-    g.elt = elt; g.out_elt = kF32; g.X = xin; g.ldx = S * H; g.W = w_pool_; g.bias = b_pool_; g.Y = pooled_;
-    g.M = B; g.N = H; g.K = H; g.epilogue = kEpiBiasTanh;
+    // pooler: first-token gather + dense + tanh on the float32 sequence output
     if (!mark(kPhPooler)) return false;
-    return launch_gemm(g, stream_);
+    return launch_pooler(x32_, w_pool_, elt, b_pool_, pooled_, B, S, H, stream_);
 }
 
 bool Model::mark(int phase) {

@@ -5,10 +5,17 @@
 // (BT/2) x (BT/2) quadrant built from 32x32 MFMA blocks.  Per K step a slab of
 // 128 bytes per row (64 bf16 / 32 f32) of both operands is loaded straight
 // from global memory into LDS (buffer_load ... lds, double buffered, one
-// barrier per step).  LDS rows are 128 bytes = eight
-// 16-byte chunks; chunk c of row r lives at position c ^ ((r ^ (r >> 3)) & 7)
-// so that the 16-byte fragment reads of 8 (or 16) consecutive rows hit
-// distinct banks.
+// barrier per step).
+//
+// LDS image of an operand tile: two sub-blocks (the two 64-byte halves of the
+// K slab), each BT rows x 64 bytes; a row is four 16-byte chunks and chunk c
+// of row r sits in slot c ^ (((r >> 1) ^ (r >> 3)) & 3), which spreads the
+// 16-byte fragment reads of 8 or 16 consecutive rows over all banks.  This is
+// also the on-device "packed" operand layout (common.h): a packed operand is
+// stored as 16 KiB blocks of 256 rows x 64 bytes that already are this image,
+// so loading a tile is a plain contiguous copy; an unpacked (row-major)
+// operand is gathered into the same image by choosing which chunk each lane
+// fetches.
 //
 // The weight tile feeds the MFMA "A" operand and the activation tile the "B"
 // operand, i.e. the hardware computes Y^T blocks: a lane then owns one token
@@ -20,8 +27,9 @@
 // the 16-byte chunk 2*kk + g of its row for both operands, so A and B always
 // pair identical k.  For f32 each chunk holds four k values consumed by four
 // 32x32x2 MFMAs; for bf16 it holds eight consumed by one 32x32x16 MFMA.
-#include <type_traits>
-
+//
+// The 256 tile in bf16 has a hand-scheduled twin (gemm_bf16_256.hip); this
+// file is the general kernel (any tile, f32, odd step counts).
 #include "gemm_common.h"
 
 namespace cubert {
@@ -32,43 +40,15 @@ namespace {
 
 using namespace gemm_detail;
 
-// Instruction order of one K step, prescribed to the machine scheduler: the
-// fragment reads of k-step 0 first, then per k-step groups of MFMAs with the
-// fragment reads of the following k-step (and, during k-step 0, the
-// global->LDS loads of the next tile) slotted in between, so that LDS and
-// memory latency run under MFMA issue instead of in front of it.
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
-
-template <int NB, int MPC>
-__device__ __forceinline__ void schedule_k_step() {
-    constexpr int RPP = NB == 4 ? 8 : (NB == 2 ? 4 : 1);      // groups per k-step
-    constexpr int MFMA_PER_GROUP = NB * NB * MPC / RPP;
-    constexpr int VMEM_PER_GROUP = 4 * NB / RPP;
-    constexpr int READS_PER_GROUP = 2 * NB / RPP;
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
-    static_for<4>([&](auto ph) {
-        static_for<RPP>([&](auto) {
-            __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER_GROUP, 0);
-            if constexpr (decltype(ph)::value == 0) __builtin_amdgcn_sched_group_barrier(0x010, VMEM_PER_GROUP, 0);
-            if constexpr (decltype(ph)::value < 3) __builtin_amdgcn_sched_group_barrier(0x100, READS_PER_GROUP, 0);
-        });
-    });
-}
-
 template <int ELT, int OUT, int EPI, int BT>
 __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     constexpr int ES = (ELT == kBF16) ? 2 : 4;       // operand element size
     constexpr int NB = BT / 64;                      // 32x32 blocks per wave and dimension
-    constexpr int GROUPS = BT / 32;                  // 8-row groups each wave moves per operand tile
-    constexpr int TILE_BYTES = BT * 128;             // one operand tile in LDS
+    constexpr int GROUPS = BT / 32;                  // loads each wave issues per operand tile and step
+    constexpr int SUB = BT * 64;                     // one sub-block (64-byte half of the K slab)
+    constexpr int TILE_BYTES = 2 * SUB;              // one operand tile in LDS
+    constexpr int SBDIV = BT / 16;                   // 16-row groups per sub-block
     constexpr int BK = 128 / ES;                     // K elements per step
-    constexpr int MPC = (ELT == kBF16) ? 1 : 4;      // MFMA instructions per 16-byte chunk pair
 
     // Two separate LDS objects (not one array indexed by parity): the compiler
     // then knows that the asynchronous global->LDS loads filling one buffer
@@ -87,24 +67,32 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     const int n0 = tile_n * BT, m0 = tile_m * BT;
 
     // ---- global -> LDS, asynchronous, no registers in between ----
-    // One buffer_load ... lds instruction moves 64 lanes x 16 bytes = 8 tile rows
-    // to 1 KiB of consecutive LDS (lane l lands at base + 16 l).  Wave w moves
-    // the 8-row groups w, w+4, w+8, ...  The LDS position (row r, slot s) must
-    // hold global chunk s ^ swz(r), so the swizzle is applied to the GLOBAL
-    // address each lane fetches from.  Rows outside the matrix (edge tiles) read
-    // as zero through the buffer descriptor's bounds check; that check covers
-    // the lane offset only, so the row part lives there and just the K offset
-    // (always in range) goes into the scalar offset.
+    // One buffer_load ... lds instruction moves 64 lanes x 16 bytes = 16 tile rows
+    // of one sub-block to 1 KiB of consecutive LDS (lane l lands at base + 16 l).
+    // The wave's i-th load handles load number q = wave + 4 i of the tile:
+    // sub-block q / SBDIV, 16-row group q % SBDIV.
+    //   unpacked source: lane fetches row 16*group + l/4 and the chunk that belongs
+    //     into LDS slot l%4, i.e. chunk (l%4) ^ swz(row); rows outside the matrix
+    //     read as zero through the buffer descriptor's bounds check (which covers
+    //     the lane offset only, so the row part lives there and just the K offset,
+    //     always in range, goes into the scalar offset);
+    //   packed source: the 1 KiB is contiguous in memory.
+    const int KB = p.K * ES / 64;                    // 64-byte blocks per packed row
     const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<unsigned char*>(p.W), 0, (int)((size_t)p.N * p.K * ES), 0x00020000);
+        const_cast<unsigned char*>(p.W), 0,
+        p.w_packed ? (int)packed_bytes(p.N, p.K * ES) : (int)((size_t)p.N * p.K * ES), 0x00020000);
     const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<unsigned char*>(p.X), 0, (int)((((size_t)p.M - 1) * p.ldx + p.K) * ES), 0x00020000);
+        const_cast<unsigned char*>(p.X), 0,
+        p.x_packed ? (int)packed_bytes(p.M, p.K * ES) : (int)((((size_t)p.M - 1) * p.ldx + p.K) * ES), 0x00020000);
     const int w_rowb = p.K * ES, x_rowb = p.ldx * ES;
-    const int dr = lane >> 3;
-    const int dc = (lane & 7) ^ dr ^ wave;          // chunk fetched for even group index; odd: dc ^ 4
-    const int w_v0 = (n0 + 8 * wave + dr) * w_rowb + (dc << 4);
-    const int x_v0 = (m0 + 8 * wave + dr) * x_rowb + (dc << 4);
-    const int flip = ((dc ^ 4) - dc) << 4;          // +64 or -64 bytes
+    const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
+    const int w_base = p.w_packed ? ((n0 >> 8) * KB * 16384 + (n0 & 255) * 64 + wave * 1024 + lane * 16)
+                                  : ((n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4));
+    const int x_base = p.x_packed ? ((m0 >> 8) * KB * 16384 + (m0 & 255) * 64 + wave * 1024 + lane * 16)
+                                  : ((m0 + 16 * wave + (lane >> 2)) * x_rowb + (dc << 4));
+    const int w_gs = p.w_packed ? 1024 : 16 * w_rowb, w_ss = p.w_packed ? 16384 : 64;   // group / sub-block strides
+    const int x_gs = p.x_packed ? 1024 : 16 * x_rowb, x_ss = p.x_packed ? 16384 : 64;
+    const int w_ks = p.w_packed ? 32768 : 128, x_ks = p.x_packed ? 32768 : 128;         // K step strides
 
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
     const int KT = p.K / BK;
@@ -114,23 +102,24 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     do {                                                                                                    \
         const int oob = (kt) < KT ? 0 : 0x40000000;                                                         \
         _Pragma("unroll") for (int i = 0; i < GROUPS; ++i) {                                                \
-            const int fl = (i & 1) ? flip : 0;                                                              \
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(wres, (lds_ptr_t)((BUF) + (wave + 4 * i) * 1024), 16,  \
-                                                     (w_v0 + fl + i * 32 * w_rowb) | oob, (kt) * 128, 0, 0); \
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (lds_ptr_t)((BUF) + TILE_BYTES + (wave + 4 * i) * 1024), \
-                                                     16, (x_v0 + fl + i * 32 * x_rowb) | oob, (kt) * 128, 0, 0); \
+            const int sb = (4 * i) / SBDIV, gq = (4 * i) % SBDIV;                                       \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                       \
+                wres, (lds_ptr_t)((BUF) + sb * SUB + (gq + wave) * 1024), 16,                               \
+                (w_base + gq * w_gs + sb * w_ss) | oob, (kt) * w_ks, 0, 0);                                 \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                       \
+                xres, (lds_ptr_t)((BUF) + TILE_BYTES + sb * SUB + (gq + wave) * 1024), 16,                  \
+                (x_base + gq * x_gs + sb * x_ss) | oob, (kt) * x_ks, 0, 0);                                 \
         }                                                                                                   \
     } while (0)
 
     // ---- fragment read addressing ----
-    // Lane (row l32, group g) of 32x32 block i reads chunk 2*kk + g of tile row
-    // base + 32 i + l32, stored at slot (2*kk + g) ^ swz(row).  swz only depends
-    // on l32 and the parity of the block index, so the byte offset is
-    //   (off0 ^ ((i & 1) << 6) ^ (kk << 5)) + i * 4096
-    // with one lane-dependent base per operand.
-    const int s0 = (l32 ^ (l32 >> 3)) & 7;
-    const int woff0 = (wn * (BT / 2) + l32) * 128 + ((g ^ s0 ^ (((wn * NB) & 1) << 2)) << 4);
-    const int xoff0 = TILE_BYTES + (wm * (BT / 2) + l32) * 128 + ((g ^ s0 ^ (((wm * NB) & 1) << 2)) << 4);
+    // Lane (row l32, group g) of 32x32 block i reads chunk 2*(kk&1) + g of row
+    // base + 32 i + l32 in sub-block kk >> 1.  swz(row) only depends on l32 (the
+    // quadrant base and 32 i do not reach the bits it uses), so the byte offset is
+    //   (off0 ^ ((kk & 1) << 5)) + (kk >> 1) * SUB + i * 2048.
+    const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
+    const int woff0 = (wn * (BT / 2) + l32) * 64 + ((g ^ sw) << 4);
+    const int xoff0 = TILE_BYTES + (wm * (BT / 2) + l32) * 64 + ((g ^ sw) << 4);
 
     f32x16_t acc[NB][NB];
 #pragma unroll
@@ -143,15 +132,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #define CUBERT_LOAD_FRAGS(BUF, kk, WF, XF)                                                                  \
     do {                                                                                                    \
         _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                      \
-            WF[i] = *reinterpret_cast<const u32x4_t*>((BUF) + (wb ^ (((i & 1) << 6) ^ ((kk) << 5))) + i * 4096); \
+            WF[i] = *reinterpret_cast<const u32x4_t*>((BUF) + (wb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + i * 2048); \
         _Pragma("unroll") for (int j = 0; j < NB; ++j)                                                      \
-            XF[j] = *reinterpret_cast<const u32x4_t*>((BUF) + (xb ^ (((j & 1) << 6) ^ ((kk) << 5))) + j * 4096); \
+            XF[j] = *reinterpret_cast<const u32x4_t*>((BUF) + (xb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + j * 2048); \
     } while (0)
 
     // One K step on buffer CUR while the loads for the next step fill NEXT.
-    // Fragments are double buffered in registers: the reads for k-step kk+1 are
-    // in flight while the MFMAs of k-step kk issue.  The empty asm keeps the
-    // compiler from hoisting (and then spilling) every per-k-step address.
+    // The empty asm keeps the compiler from hoisting (and then spilling) every
+    // per-k-step address.
 #define CUBERT_K_STEP(CUR, NEXT, kt)                                                                        \
     do {                                                                                                    \
         CUBERT_ISSUE_TILE(NEXT, (kt) + 1);                                                                  \
@@ -165,7 +153,6 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
                 _Pragma("unroll") for (int j = 0; j < NB; ++j)                                              \
                     mfma_chunk<ELT>(wf[kk & 1][i], xf[kk & 1][j], acc[i][j]);                               \
         }                                                                                                   \
-        schedule_k_step<NB, MPC>();                                                                         \
         __builtin_amdgcn_sched_barrier(0);  /* nothing moves across the end of the step */                  \
         __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): my share of NEXT has landed */                     \
         __syncthreads();                                                                                    \
@@ -235,9 +222,11 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0 || p.K <= 0) { set_error("gemm: empty problem"); return false; }
     if (p.K % bk != 0) { set_error("gemm: K must be a multiple of " + std::to_string(bk)); return false; }
     if (p.N % 4 != 0) { set_error("gemm: N must be a multiple of 4"); return false; }
-    if (p.ldx < p.K || (p.ldx * es) % 16 != 0) { set_error("gemm: bad ldx"); return false; }
+    if (!p.x_packed && (p.ldx < p.K || (p.ldx * es) % 16 != 0)) { set_error("gemm: bad ldx"); return false; }
+    if (p.x_packed && p.ldx != p.K) { set_error("gemm: a packed X has no row stride"); return false; }
     if (!p.X || !p.W || !p.bias) { set_error("gemm: null operand"); return false; }
-    if (((size_t)p.M + 256) * p.ldx * es >= (1ull << 31) || ((size_t)p.N + 256) * p.K * es >= (1ull << 31)) {
+    if (((size_t)p.M + 256) * (p.x_packed ? p.K : p.ldx) * es >= (1ull << 31) ||
+        ((size_t)p.N + 256) * p.K * es >= (1ull << 31)) {
         set_error("gemm: operand exceeds the 2 GiB addressable through one buffer descriptor");
         return false;
     }
@@ -252,6 +241,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     d.bias = p.bias;
     d.Y = static_cast<unsigned char*>(p.Y);
     d.M = p.M; d.N = p.N; d.K = p.K; d.ldx = p.ldx;
+    d.x_packed = p.x_packed; d.w_packed = p.w_packed; d.y_packed = p.y_packed;
     int out = p.out_elt;
     if (p.epilogue == kEpiQKV) {
         if (!p.q || !p.k || !p.vt || p.S <= 0 || p.heads <= 0 || p.N != 3 * p.heads * 64 ||
@@ -263,16 +253,21 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         d.k = static_cast<unsigned char*>(p.k);
         d.vt = static_cast<unsigned char*>(p.vt);
         d.S = p.S; d.Sp = p.Sp; d.heads = p.heads; d.hidden = p.heads * 64;
+        d.y_packed = 0;
         out = p.elt;
     } else {
         if (!p.Y || (reinterpret_cast<uintptr_t>(p.Y) & 15)) { set_error("gemm: bad Y"); return false; }
         if (out != kBF16 && out != kF32) { set_error("gemm: bad output type"); return false; }
+        if (p.y_packed && (out != kBF16 || p.N % 32 != 0)) {
+            set_error("gemm: a packed Y must be bf16 with N a multiple of 32");
+            return false;
+        }
     }
     const int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N);
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
     if (p.elt == kBF16) {
-        // 256 tile with an even number of K steps: the hand-scheduled kernel
+        // 256 tile with a multiple of four half-steps: the hand-scheduled kernel
         if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled)
             return launch_gemm_bf16_t256(d, out, p.epilogue, stream);
         return out == kBF16 ? launch_epi<kBF16, kBF16>(d, p.epilogue, bt, stream)

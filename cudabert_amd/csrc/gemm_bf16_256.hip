@@ -15,10 +15,10 @@ namespace {
 using namespace gemm_detail;
 
 #define CUBERT_ACC_OPERANDS                                                                              \
-    [c00] "+a"(acc[0][0]), [c01] "+a"(acc[0][1]), [c02] "+a"(acc[0][2]), [c03] "+a"(acc[0][3]),         \
-    [c10] "+a"(acc[1][0]), [c11] "+a"(acc[1][1]), [c12] "+a"(acc[1][2]), [c13] "+a"(acc[1][3]),         \
-    [c20] "+a"(acc[2][0]), [c21] "+a"(acc[2][1]), [c22] "+a"(acc[2][2]), [c23] "+a"(acc[2][3]),         \
-    [c30] "+a"(acc[3][0]), [c31] "+a"(acc[3][1]), [c32] "+a"(acc[3][2]), [c33] "+a"(acc[3][3])
+    [c00] "=&a"(acc[0][0]), [c01] "=&a"(acc[0][1]), [c02] "=&a"(acc[0][2]), [c03] "=&a"(acc[0][3]),         \
+    [c10] "=&a"(acc[1][0]), [c11] "=&a"(acc[1][1]), [c12] "=&a"(acc[1][2]), [c13] "=&a"(acc[1][3]),         \
+    [c20] "=&a"(acc[2][0]), [c21] "=&a"(acc[2][1]), [c22] "=&a"(acc[2][2]), [c23] "=&a"(acc[2][3]),         \
+    [c30] "=&a"(acc[3][0]), [c31] "=&a"(acc[3][1]), [c32] "=&a"(acc[3][2]), [c33] "=&a"(acc[3][3])
 
 #define CUBERT_V10(b) "v" #b "0", "v" #b "1", "v" #b "2", "v" #b "3", "v" #b "4", "v" #b "5", "v" #b "6", "v" #b "7", "v" #b "8", "v" #b "9"
 
@@ -42,39 +42,45 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     // Rows outside the matrix read as zero (bounds check on the lane offset).
     const unsigned long long wa = reinterpret_cast<unsigned long long>(p.W);
     const unsigned long long xa = reinterpret_cast<unsigned long long>(p.X);
-    const u32x4_t wres = {(unsigned)wa, (unsigned)(wa >> 32) & 0xffffu, (unsigned)((size_t)p.N * p.K * 2), 0x00020000u};
-    const u32x4_t xres = {(unsigned)xa, (unsigned)(xa >> 32) & 0xffffu,
-                          (unsigned)((((size_t)p.M - 1) * p.ldx + p.K) * 2), 0x00020000u};
+    const unsigned wsize = p.w_packed ? (unsigned)packed_bytes(p.N, (size_t)p.K * 2) : (unsigned)((size_t)p.N * p.K * 2);
+    const unsigned xsize = p.x_packed ? (unsigned)packed_bytes(p.M, (size_t)p.K * 2)
+                                      : (unsigned)((((size_t)p.M - 1) * p.ldx + p.K) * 2);
+    const u32x4_t wres = {(unsigned)wa, (unsigned)(wa >> 32) & 0xffffu, wsize, 0x00020000u};
+    const u32x4_t xres = {(unsigned)xa, (unsigned)(xa >> 32) & 0xffffu, xsize, 0x00020000u};
     const int w_rowb = p.K * 2, x_rowb = p.ldx * 2;
-    // global->LDS: one load moves 16 rows; lane fetches row 16*group + lane/4 and the chunk
-    // that belongs into its LDS slot lane%4 (slot = chunk ^ swz(row)).  Wave w moves the
-    // groups w, w+4, w+8, w+12, for which swz only depends on the lane and the parity of w.
+    const int KB = p.K * 2 / 64;
+    // global->LDS: one load moves 16 rows x 64 bytes.  Wave w moves the row groups w, w+4,
+    // w+8, w+12 of each tile.
+    //   unpacked source: lane fetches row 16*group + lane/4 and the chunk that belongs into
+    //     its LDS slot lane%4 (slot = chunk ^ swz(row)); for these groups swz only depends on
+    //     the lane and the parity of w.  One half-step further along K is +64 bytes.
+    //   packed source: a tile's half-step is one contiguous 16 KiB block, the next one follows it.
     const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
-    const int w_v0 = (n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4);
-    const int x_v0 = (m0 + 16 * wave + (lane >> 2)) * x_rowb + (dc << 4);
-    const int w64 = 64 * w_rowb, x64 = 64 * x_rowb;
+    const int w_v0 = p.w_packed ? (tile_n * KB * 16384 + wave * 1024 + lane * 16)
+                                : ((n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4));
+    const int x_v0 = p.x_packed ? (tile_m * KB * 16384 + wave * 1024 + lane * 16)
+                                : ((m0 + 16 * wave + (lane >> 2)) * x_rowb + (dc << 4));
+    const int w64 = p.w_packed ? 4096 : 64 * w_rowb, x64 = p.x_packed ? 4096 : 64 * x_rowb;
+    const int wkstep = p.w_packed ? 16384 : 64, xkstep = p.x_packed ? 16384 : 64;
     // fragment reads: chunk g of my row in the W / X tile of stage 0, k-phase 0
     const int lds_base = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
     const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
     const int wb = lds_base + (wn * 128 + l32) * 64 + ((g ^ sw) << 4);
     const int xb = lds_base + 16384 + (wm * 128 + l32) * 64 + ((g ^ sw) << 4);
-    const int m0b = lds_base + wave * 1024;
+    const int m0b = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
+    const int ldsw = lds_base + wave * 1024 + lane * 16;      // where my 16 bytes of a loaded row group go
     const int ht = p.K / 32;          // half-steps; a multiple of 4
 
-    f32x16_t acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    f32x16_t acc[4][4];       // zeroed inside the asm block
 
     asm volatile(
 #include "gemm_bf16_256_loop.inc"
         : CUBERT_ACC_OPERANDS
         : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
-          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b)
-        : "memory", "scc", "s92", "s93", "s94", "s95", "s96", "s97", "v176", "v177", "v178", "v179",
+          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep),
+          [ldsw] "v"(ldsw)
+        : "memory", "scc", "s92", "s93", "s94", "s95", "s96", "s97", "s98", CUBERT_V10(10), CUBERT_V10(11), CUBERT_V10(12), CUBERT_V10(13), CUBERT_V10(14), CUBERT_V10(15),
+          "v160", "v161", "v162", "v163", "v170", "v171", "v176", "v177", "v178", "v179",
           CUBERT_V10(18), CUBERT_V10(19), CUBERT_V10(20), CUBERT_V10(21), CUBERT_V10(22), CUBERT_V10(23),
           CUBERT_V10(24), "v250", "v251", "v252", "v253", "v254", "v255");
 

@@ -23,6 +23,7 @@ struct GemmDev {
     int M, N, K, ldx;
     int S, Sp, heads, hidden;
     int tiles_n, tiles_m;
+    int x_packed, w_packed, y_packed;     // operand / result in the packed layout (common.h)
 };
 
 __device__ __forceinline__ float gelu_erf(float x) {
@@ -130,6 +131,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                     } else {
                         store4<OUT>(which == 0 ? p.q : p.k, (bh * p.S + sidx) * 64 + dd, v);
                     }
+                } else if (p.y_packed) {
+                    // packed bf16 result: the next GEMM's activation operand
+                    bf16x4_t o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+                    *reinterpret_cast<bf16x4_t*>(p.Y + packed_offset(m, n * 2, p.N * 2 / 64)) = o;
                 } else {
                     store4<OUT>(p.Y, (size_t)m * p.N + n, v);
                 }

@@ -43,6 +43,8 @@ struct GemmParams {
     int S = 0, Sp = 0, heads = 0;
     int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile)
     bool compiler_scheduled = false;   // 256 tile: use the generic kernel, not the hand-scheduled one
+    // Packed operand layout (common.h): X / W read from it, Y (bf16, plain epilogues) written in it.
+    bool x_packed = false, w_packed = false, y_packed = false;
 };
 bool launch_gemm(const GemmParams& p, hipStream_t stream);
 
@@ -54,8 +56,9 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream);
 // Replaces Query_Key / op_SoftMax / Prob_Value of the reference
 // (cuda_bert/ops/batch_matmul.cu:48-83,107-141; ops/softmax.cu:86-143)
 // without materialising the [B,S,heads,S] score tensor.
+// ctx_packed (bf16 only): write ctx in the packed GEMM-operand layout (common.h).
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd,
-                      void* ctx, int B, int heads, int S, int Sp, float scale, int elt,
+                      void* ctx, bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt,
                       hipStream_t stream);
 
 // ----------------------------------------------------------- LayerNorm -----
@@ -64,8 +67,10 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
 // written as the next GEMM's operand.  y has type y_elt (may be nullptr: plain
 // LayerNorm).  eps = 1e-12 inside the square root, biased variance
 // (cuda_bert/ops/layernorm.cu:136-182; modeling.py:168-172).
+// xb_packed: write the copy in the packed GEMM-operand layout (common.h).
 bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
-                          const float* beta, bf16_t* xb, int rows, int H, hipStream_t stream);
+                          const float* beta, bf16_t* xb, bool xb_packed, int rows, int H,
+                          hipStream_t stream);
 
 // --------------------------------------------------- embedding + LN --------
 // x[t] = LayerNorm(word[ids[t]] + pos[t % S] + type[seg[t]]); also writes the
@@ -74,8 +79,8 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
 // (cuda_bert/ops/embedding.cu:3-58; utils/bert.cu:94-97 for the positions.)
 bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
                             const float* pos, const float* type, const float* gamma,
-                            const float* beta, float* x, bf16_t* xb, float* maskadd, int B, int S,
-                            int Sp, int H, int vocab, int type_vocab, hipStream_t stream);
+                            const float* beta, float* x, bf16_t* xb, bool xb_packed, float* maskadd,
+                            int B, int S, int Sp, int H, int vocab, int type_vocab, hipStream_t stream);
 
 // ------------------------------------------------ scale+mask+softmax -------
 // In place over materialised scores [B, rows_per_batch, S] (float32 or bf16):
@@ -90,9 +95,19 @@ bool launch_mask_softmax(void* scores, int elt, const int* mask, int B, int rows
 bool launch_classifier(const float* pooled, const float* kernel, const float* bias, float* probs,
                        int B, int H, int C, hipStream_t stream);
 
+// ------------------------------------------------------------ pooler -------
+// pooled[b, :] = tanh(x[b * S, :] @ W^T + bias): first-token gather + dense +
+// tanh in one kernel; x is the float32 sequence output [B*S, H], W [H, H]
+// row-major ([out, in]) of type w_elt (cuda_bert/ops/elementwise.cu:5-32, 56-70 and
+// the pooler op_Linear of cuda_bert/utils/bert.cu:238-247; modeling.py:347-353).
+bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, float* pooled, int B, int S, int H,
+                   hipStream_t stream);
+
 // ------------------------------------------------------ load helpers -------
-// dst[n, k] = convert(src[k, n])  : on-disk [in,out] float32 -> [out,in] operand type.
-bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt,
+// dst[n, k] = convert(src[k, n])  : on-disk [in,out] float32 -> [out,in] operand type,
+// row-major or (bf16) packed; in the packed case dst is the whole operand and the
+// tensor's rows land at row0 .. row0 + N - 1 of it.
+bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt, bool packed, int row0,
                               hipStream_t stream);
 bool launch_fill_f32(float* dst, float value, size_t n, hipStream_t stream);
 

@@ -25,10 +25,12 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // Normalises the row held in v[][] (lane owns elements c*256 + lane*4 + e) and
 // writes it to x (f32) and optionally xb (bf16).
+// xb (optional) receives the bf16 copy: row-major when xb_packed == 0, else in
+// the packed GEMM-operand layout (common.h).
 __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H, int lane,
                                                 const float* __restrict__ gamma,
                                                 const float* __restrict__ beta, float* xrow,
-                                                bf16_t* xbrow) {
+                                                bf16_t* xb, int row, int xb_packed) {
     float s = 0.0f;
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c)
@@ -56,9 +58,11 @@ __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[e] = g4[e] * (v[c][e] * rstd) + b4[e];
             *reinterpret_cast<f32x4_t*>(xrow + i) = o;
-            if (xbrow) {
+            if (xb) {
                 bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
-                *reinterpret_cast<bf16x4_t*>(xbrow + i) = ob;
+                unsigned char* dst = reinterpret_cast<unsigned char*>(xb);
+                const size_t off = xb_packed ? packed_offset(row, i * 2, H * 2 / 64) : ((size_t)row * H + i) * 2;
+                *reinterpret_cast<bf16x4_t*>(dst + off) = ob;
             }
         }
     }
@@ -69,7 +73,8 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
                                                             const unsigned char* __restrict__ y,
                                                             const float* __restrict__ gamma,
                                                             const float* __restrict__ beta,
-                                                            bf16_t* __restrict__ xb, int rows, int H) {
+                                                            bf16_t* __restrict__ xb, int rows, int H,
+                                                            int xb_packed) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -92,7 +97,7 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
             for (int e = 0; e < 4; ++e) v[c][e] = a[e];
         }
     }
-    normalise_store(v, H, lane, gamma, beta, xrow, xb ? xb + (size_t)row * H : nullptr);
+    normalise_store(v, H, lane, gamma, beta, xrow, xb, row, xb_packed);
 }
 
 __global__ __launch_bounds__(256) void embed_layernorm_kernel(
@@ -100,7 +105,7 @@ __global__ __launch_bounds__(256) void embed_layernorm_kernel(
     const float* __restrict__ word, const float* __restrict__ pos, const float* __restrict__ type,
     const float* __restrict__ gamma, const float* __restrict__ beta, float* __restrict__ x,
     bf16_t* __restrict__ xb, float* __restrict__ maskadd, int B, int S, int Sp, int H, int vocab,
-    int type_vocab) {
+    int type_vocab, int xb_packed) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= B * S) return;
@@ -130,7 +135,7 @@ __global__ __launch_bounds__(256) void embed_layernorm_kernel(
             for (int e = 0; e < 4; ++e) v[c][e] = (a[e] + p4[e]) + t4[e];
         }
     }
-    normalise_store(v, H, lane, gamma, beta, x + (size_t)row * H, xb ? xb + (size_t)row * H : nullptr);
+    normalise_store(v, H, lane, gamma, beta, x + (size_t)row * H, xb, row, xb_packed);
 }
 
 // One wave per score row of length S <= 512 (8 elements per lane, strided by
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(64) void classifier_kernel(const float* __restrict_
 template <int ELT>
 __global__ __launch_bounds__(256) void transpose_convert_kernel(const float* __restrict__ src,
                                                                 unsigned char* __restrict__ dst, int K,
-                                                                int N) {
+                                                                int N, int packed, int row0) {
     __shared__ float tile[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;      // 32 x 8
     const int n0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
@@ -232,8 +237,12 @@ __global__ __launch_bounds__(256) void transpose_convert_kernel(const float* __r
         const int nn = n0 + r, kk = k0 + tx;
         if (nn < N && kk < K) {
             const float val = tile[tx][r];
-            if constexpr (ELT == kBF16) reinterpret_cast<__bf16*>(dst)[(size_t)nn * K + kk] = (__bf16)val;
-            else reinterpret_cast<float*>(dst)[(size_t)nn * K + kk] = val;
+            if constexpr (ELT == kBF16) {
+                const size_t off = packed ? packed_offset(row0 + nn, kk * 2, K * 2 / 64) : ((size_t)nn * K + kk) * 2;
+                *reinterpret_cast<__bf16*>(dst + off) = (__bf16)val;
+            } else {
+                reinterpret_cast<float*>(dst)[(size_t)nn * K + kk] = val;
+            }
         }
     }
 }
@@ -243,12 +252,59 @@ __global__ void fill_f32_kernel(float* dst, float value, size_t n) {
         dst[i] = value;
 }
 
+// pooled[b, n] = tanh(bias[n] + sum_k x[b * S, k] * W[n, k]): the first-token
+// gather (row stride S*H of the float32 sequence output), the dense layer and
+// the tanh in one pass.  A workgroup handles one batch row and 64 outputs; each
+// wave 16 outputs, lanes split K.  W is [H, H] row-major ([out, in]).
+template <int ELT>
+__global__ __launch_bounds__(256) void pooler_kernel(const float* __restrict__ x, const unsigned char* __restrict__ W,
+                                                     const float* __restrict__ bias, float* __restrict__ pooled,
+                                                     int S, int H) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.x;
+    const float* xr = x + (size_t)b * S * H;
+    float xv[kMaxChunks][4];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+        const int i = c * 256 + lane * 4;
+        if (i < H) {
+            const f32x4_t t = *reinterpret_cast<const f32x4_t*>(xr + i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xv[c][e] = t[e];
+        }
+    }
+    for (int o = 0; o < 16; ++o) {
+        const int n = blockIdx.y * 64 + wave * 16 + o;
+        if (n >= H) break;
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c) {
+            const int i = c * 256 + lane * 4;
+            if (i < H) {
+                if constexpr (ELT == kBF16) {
+                    const bf16x4_t w4 = *reinterpret_cast<const bf16x4_t*>(W + ((size_t)n * H + i) * 2);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc += xv[c][e] * (float)w4[e];
+                } else {
+                    const f32x4_t w4 = *reinterpret_cast<const f32x4_t*>(W + ((size_t)n * H + i) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc += xv[c][e] * w4[e];
+                }
+            }
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) pooled[(size_t)b * H + n] = tanhf(acc + bias[n]);
+    }
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
 
 bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta,
-                          bf16_t* xb, int rows, int H, hipStream_t stream) {
+                          bf16_t* xb, bool xb_packed, int rows, int H, hipStream_t stream) {
+    if (xb && xb_packed && H % 32 != 0) { set_error("layernorm: a packed copy needs H to be a multiple of 32"); return false; }
+    const int xp = xb_packed ? 1 : 0;
     if (rows <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
         set_error("layernorm: H must be a multiple of 4 and at most 1024");
         return false;
@@ -260,9 +316,9 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
     }
     dim3 grid((rows + 3) / 4), block(256);
     const unsigned char* yc = static_cast<const unsigned char*>(y);
-    if (!y) hipLaunchKernelGGL(add_layernorm_kernel<-1>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H);
-    else if (y_elt == kF32) hipLaunchKernelGGL(add_layernorm_kernel<kF32>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H);
-    else if (y_elt == kBF16) hipLaunchKernelGGL(add_layernorm_kernel<kBF16>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H);
+    if (!y) hipLaunchKernelGGL(add_layernorm_kernel<-1>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp);
+    else if (y_elt == kF32) hipLaunchKernelGGL(add_layernorm_kernel<kF32>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp);
+    else if (y_elt == kBF16) hipLaunchKernelGGL(add_layernorm_kernel<kBF16>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp);
     else { set_error("layernorm: bad addend type"); return false; }
     CUBERT_HIP_OK(hipGetLastError());
     return true;
@@ -270,8 +326,9 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
 
 bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
                             const float* pos, const float* type, const float* gamma, const float* beta,
-                            float* x, bf16_t* xb, float* maskadd, int B, int S, int Sp, int H, int vocab,
-                            int type_vocab, hipStream_t stream) {
+                            float* x, bf16_t* xb, bool xb_packed, float* maskadd, int B, int S, int Sp, int H,
+                            int vocab, int type_vocab, hipStream_t stream) {
+    if (xb && xb_packed && H % 32 != 0) { set_error("embedding: a packed copy needs H to be a multiple of 32"); return false; }
     if (B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
         set_error("embedding: H must be a multiple of 4 and at most 1024");
         return false;
@@ -289,7 +346,7 @@ bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, con
     const long rows = (long)B * S;
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
     hipLaunchKernelGGL(embed_layernorm_kernel, grid, block, 0, stream, ids, seg, mask, word, pos, type, gamma,
-                       beta, x, xb, maskadd, B, S, Sp, H, vocab, type_vocab);
+                       beta, x, xb, maskadd, B, S, Sp, H, vocab, type_vocab, xb_packed ? 1 : 0);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }
@@ -322,12 +379,32 @@ bool launch_classifier(const float* pooled, const float* kernel, const float* bi
     return true;
 }
 
-bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt, hipStream_t stream) {
+bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, float* pooled, int B, int S, int H,
+                   hipStream_t stream) {
+    if (B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
+        set_error("pooler: H must be a multiple of 4 and at most 1024");
+        return false;
+    }
+    if (!x || !W || !bias || !pooled || !aligned16(x) || !aligned16(W)) { set_error("pooler: null or misaligned operand"); return false; }
+    if (B > 65535) { set_error("pooler: batch too large"); return false; }
+    dim3 grid(B, (H + 63) / 64), block(256);
+    const unsigned char* wc = static_cast<const unsigned char*>(W);
+    if (w_elt == kBF16) hipLaunchKernelGGL(pooler_kernel<kBF16>, grid, block, 0, stream, x, wc, bias, pooled, S, H);
+    else if (w_elt == kF32) hipLaunchKernelGGL(pooler_kernel<kF32>, grid, block, 0, stream, x, wc, bias, pooled, S, H);
+    else { set_error("pooler: bad weight type"); return false; }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt, bool packed, int row0,
+                              hipStream_t stream) {
     if (!src || !dst || K <= 0 || N <= 0) { set_error("transpose: bad arguments"); return false; }
+    if (packed && (elt != kBF16 || K % 32 != 0)) { set_error("transpose: packed output is bf16 with K a multiple of 32"); return false; }
+    const int pk = packed ? 1 : 0;
     dim3 grid((N + 31) / 32, (K + 31) / 32), block(256);
     unsigned char* d = static_cast<unsigned char*>(dst);
-    if (elt == kBF16) hipLaunchKernelGGL(transpose_convert_kernel<kBF16>, grid, block, 0, stream, src, d, K, N);
-    else if (elt == kF32) hipLaunchKernelGGL(transpose_convert_kernel<kF32>, grid, block, 0, stream, src, d, K, N);
+    if (elt == kBF16) hipLaunchKernelGGL(transpose_convert_kernel<kBF16>, grid, block, 0, stream, src, d, K, N, pk, row0);
+    else if (elt == kF32) hipLaunchKernelGGL(transpose_convert_kernel<kF32>, grid, block, 0, stream, src, d, K, N, pk, row0);
     else { set_error("transpose: bad element type"); return false; }
     CUBERT_HIP_OK(hipGetLastError());
     return true;

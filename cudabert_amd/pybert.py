@@ -89,18 +89,25 @@ for _n in ("cubert_hidden_size", "cubert_num_classes", "cubert_precision", "cube
 lib.cubert_capacity_tokens.argtypes = [c_void_p]
 lib.cubert_capacity_tokens.restype = c_long
 
+X_PACKED, W_PACKED, Y_PACKED, COMPILER_SCHEDULED = 1, 2, 4, 8      # layout flags of the op entry points
+lib.cubert_packed_bytes.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+lib.cubert_packed_bytes.restype = ctypes.c_size_t
+lib.cubert_packed_offset.argtypes = [c_int, c_int, c_int]
+lib.cubert_packed_offset.restype = ctypes.c_size_t
 lib.cubert_op_gemm.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                               c_int, c_int, c_void_p]
+                               c_int, c_int, c_int, c_void_p]
 lib.cubert_op_gemm.restype = c_int
-lib.cubert_op_gemm_qkv.argtypes = [c_void_p] * 6 + [c_int] * 5 + [c_void_p]
+lib.cubert_op_gemm_qkv.argtypes = [c_void_p] * 6 + [c_int] * 6 + [c_void_p]
 lib.cubert_op_gemm_qkv.restype = c_int
-lib.cubert_op_attention.argtypes = [c_void_p] * 5 + [c_int, c_int, c_int, c_float, c_int, c_void_p]
+lib.cubert_op_attention.argtypes = [c_void_p] * 5 + [c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]
 lib.cubert_op_attention.restype = c_int
 lib.cubert_op_add_layernorm.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                                        c_void_p]
+                                        c_int, c_void_p]
 lib.cubert_op_add_layernorm.restype = c_int
-lib.cubert_op_embed_layernorm.argtypes = [c_void_p] * 11 + [c_int] * 5 + [c_void_p]
+lib.cubert_op_embed_layernorm.argtypes = [c_void_p] * 11 + [c_int] * 6 + [c_void_p]
 lib.cubert_op_embed_layernorm.restype = c_int
+lib.cubert_op_pooler.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+lib.cubert_op_pooler.restype = c_int
 lib.cubert_op_mask_softmax.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]
 lib.cubert_op_mask_softmax.restype = c_int
 

@@ -132,35 +132,55 @@ long cubert_capacity_tokens(void* model);
  * timing).  `stream` is a hipStream_t (NULL = default stream); elt: 0 float32,
  * 1 bfloat16.  All return 0 on success. ---- */
 
+/* Layout flags of the GEMM entry points.  A "packed" operand is stored as
+ * 16 KiB blocks of 256 rows x 64 bytes in the order the kernels' LDS tiles use
+ * (cubert_packed_bytes / cubert_packed_offset give size and element address);
+ * in bf16 mode the engine keeps weights and GEMM-input activations this way. */
+#define CUBERT_X_PACKED 1           /* activation operand X is packed */
+#define CUBERT_W_PACKED 2           /* weight operand W is packed */
+#define CUBERT_Y_PACKED 4           /* write Y packed (bf16 output only) */
+#define CUBERT_COMPILER_SCHEDULED 8 /* 256 tile: general kernel instead of the hand-scheduled one */
+size_t cubert_packed_bytes(size_t rows, size_t row_bytes);
+size_t cubert_packed_offset(int row, int byte_in_row, int row_bytes);
+
 /* Y[M,N] = epilogue(X[M,K] (row stride ldx) * W[N,K]^T + bias[N]);
  * epilogue 0 bias, 1 bias+GELU(erf), 2 bias+tanh.  tile 0 = automatic.
  * Replaces op_Linear::forward (cuda_bert/ops/linear.cu:91-148) + op_Gelu /
  * op_Tanh (ops/elementwise.cu:37-70). */
 int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int M, int N, int K,
-                   int ldx, int elt, int out_elt, int epilogue, int tile, void* stream);
+                   int ldx, int elt, int out_elt, int epilogue, int tile, int flags, void* stream);
 
 /* Fused QKV projection (op_BatchedLinear::forward, cuda_bert/ops/linear.cu:241-319):
  * X[B*S, hidden] * Wqkv[3*hidden, hidden]^T + bias -> q,k [B,heads,S,64],
  * vt [B,heads,64,Sp] with Sp = S rounded up to 32. */
 int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q, void* k, void* vt,
-                       int B, int S, int heads, int elt, int tile, void* stream);
+                       int B, int S, int heads, int elt, int tile, int flags, void* stream);
 
 /* Fused attention (Query_Key + op_SoftMax + Prob_Value,
  * cuda_bert/ops/batch_matmul.cu:48-141, ops/softmax.cu:86-143). */
 int cubert_op_attention(const void* q, const void* k, const void* vt, const float* maskadd,
-                        void* ctx, int B, int heads, int S, float scale, int elt, void* stream);
+                        void* ctx, int B, int heads, int S, float scale, int elt, int flags,
+                        void* stream); /* flags: CUBERT_Y_PACKED writes ctx packed (bf16) */
 
 /* x <- LayerNorm(x + y); optional bf16 copy xb (op_LayerNorm::forward,
  * cuda_bert/ops/layernorm.cu:136-206). */
 int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
-                            const float* beta, void* xb, int rows, int hidden, void* stream);
+                            const float* beta, void* xb, int rows, int hidden, int flags,
+                            void* stream); /* flags: CUBERT_Y_PACKED writes xb packed */
 
 /* Embedding gather + add + LayerNorm + additive mask rows (Embedding::forward,
  * cuda_bert/ops/embedding.cu:3-58). */
 int cubert_op_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
                               const float* pos, const float* type, const float* gamma,
                               const float* beta, float* x, void* xb, float* maskadd, int B, int S,
-                              int hidden, int vocab, int type_vocab, void* stream);
+                              int hidden, int vocab, int type_vocab, int flags, void* stream);
+
+/* pooled[b, :] = tanh(x[b * S, :] @ W^T + bias): first-token gather, dense and
+ * tanh in one kernel (copy_pooler + op_Linear + op_Tanh, cuda_bert/utils/bert.cu:238-247;
+ * ops/elementwise.cu:5-32, 56-70).  x float32 [B*S, hidden], W [hidden, hidden]
+ * row-major ([out, in]) of type w_elt. */
+int cubert_op_pooler(const float* x, const void* W, const float* bias, float* pooled, int B, int S,
+                     int hidden, int w_elt, void* stream);
 
 /* In-place scale + mask + softmax over materialised scores [B, rows_per_batch, S]
  * (cuApplySoftmax, cuda_bert/ops/softmax.cu:86-143). */

@@ -33,6 +33,43 @@ def bf16_round(a):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(torch.float32).numpy()
 
 
+def pack_p64(a_u16):
+    """Row-major [R, K] 16-bit array -> packed GEMM-operand layout (flat uint16)."""
+    R, K = a_u16.shape
+    row_bytes = K * 2
+    KB = row_bytes // 64
+    out = np.zeros(((R + 255) // 256) * KB * 8192, np.uint16)
+    out[packed_index(R, K)] = a_u16
+    return out
+
+
+def packed_index(R, K):
+    """uint16 index of element (r, k) in the packed layout; checked against the library's own formula."""
+    r = np.arange(R)[:, None]
+    kbyte = (np.arange(K) * 2)[None, :]
+    KB = K * 2 // 64
+    rp = r & 255
+    sw = ((rp >> 1) ^ (rp >> 3)) & 3
+    off = ((r >> 8) * KB + (kbyte >> 6)) * 16384 + rp * 64 + ((((kbyte >> 4) & 3) ^ sw) << 4) + (kbyte & 15)
+    return off // 2
+
+
+def bf16_bits(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+
+
+def bits_to_f32(u16):
+    return torch.from_numpy(u16.view(np.int16).copy()).view(torch.bfloat16).float().numpy()
+
+
+def test_packed_offset_formula(pb):
+    idx = packed_index(300, 128)
+    for r, k in ((0, 0), (1, 9), (17, 40), (255, 127), (256, 0), (299, 77)):
+        assert pb.lib.cubert_packed_offset(r, k * 2, 256) == idx[r, k] * 2
+    assert pb.lib.cubert_packed_bytes(300, 256) == 2 * 4 * 16384
+    assert len(np.unique(idx)) == idx.size
+
+
 def gelu64(x):
     from scipy.special import erf
     return x * 0.5 * (1.0 + erf(x / math.sqrt(2.0)))
@@ -60,7 +97,7 @@ def test_gemm(pb, elt, tile, M, N, K, epi):
         Xd, Wd, bd = dev(X, tdt), dev(W, tdt), dev(b)
         Y = torch.full((M, N), float("nan"), dtype=torch.float32 if out_elt == F32 else torch.bfloat16, device="cuda")
         pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), M, N, K, K, elt,
-                                       out_elt, epi, tile, stream()))
+                                       out_elt, epi, tile, 0, stream()))
         torch.cuda.synchronize()
         got = Y.float().cpu().numpy().astype(np.float64)
         tol = 2e-4 if out_elt == F32 else 2e-2 * max(1.0, np.abs(ref).max() / 4)
@@ -79,7 +116,7 @@ def test_gemm_strided_rows(pb):
     Xd, Wd, bd = dev(seq), dev(W), dev(b)
     Y = torch.zeros((B, H), device="cuda")
     pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), B, H, H, S * H, F32, F32,
-                                   2, 0, stream()))
+                                   2, 0, 0, stream()))
     torch.cuda.synchronize()
     assert np.abs(Y.cpu().numpy() - ref).max() < 1e-4
 
@@ -90,10 +127,10 @@ def test_gemm_rejects_bad_shapes(pb):
     b = torch.zeros(64, device="cuda")
     Y = torch.zeros((64, 64), device="cuda")
     rc = pb.lib.cubert_op_gemm(X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), 64, 64, 96, 96, BF16, F32, 0, 0,
-                               stream())
+                               0, stream())
     assert rc != 0 and "multiple of 64" in pb.last_error()
     rc = pb.lib.cubert_op_gemm(X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), 64, 64, 96, 96, F32, F32, 0, 99,
-                               stream())
+                               0, stream())
     assert rc != 0
 
 
@@ -119,7 +156,7 @@ def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile):
     k = torch.zeros_like(q)
     vt = torch.zeros((B, heads, 64, Sp), dtype=tdt, device="cuda")
     pb.check(pb.lib.cubert_op_gemm_qkv(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), q.data_ptr(), k.data_ptr(),
-                                       vt.data_ptr(), B, S, heads, elt, tile, stream()))
+                                       vt.data_ptr(), B, S, heads, elt, tile, 0, stream()))
     torch.cuda.synchronize()
     tol = 2e-4 if elt == F32 else 3e-2
     assert np.abs(q.float().cpu().numpy() - q_ref).max() < tol
@@ -158,7 +195,7 @@ def test_attention(pb, elt, B, S, heads):
     qd, kd, vd, md = dev(q, tdt), dev(k, tdt), dev(vt, tdt), dev(maskadd)
     ctx = torch.full((B * S, heads * 64), float("nan"), dtype=tdt, device="cuda")
     pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), ctx.data_ptr(),
-                                        B, heads, S, scale, elt, stream()))
+                                        B, heads, S, scale, elt, 0, stream()))
     torch.cuda.synchronize()
     got = ctx.float().cpu().numpy()
     assert np.isfinite(got).all()
@@ -185,7 +222,7 @@ def test_add_layernorm(pb, H, y_elt):
     yd = None if y_elt is None else dev(y, torch.float32 if y_elt == F32 else torch.bfloat16)
     xb = torch.zeros((rows, H), dtype=torch.bfloat16, device="cuda")
     pb.check(pb.lib.cubert_op_add_layernorm(xd.data_ptr(), None if yd is None else yd.data_ptr(), y_elt or 0,
-                                            gd.data_ptr(), bd.data_ptr(), xb.data_ptr(), rows, H, stream()))
+                                            gd.data_ptr(), bd.data_ptr(), xb.data_ptr(), rows, H, 0, stream()))
     torch.cuda.synchronize()
     got = xd.cpu().numpy()
     assert np.abs(got - ref).max() < 2e-5
@@ -213,7 +250,7 @@ def test_embed_layernorm(pb):
     madd = torch.zeros((B, Sp), device="cuda")
     args = [dev(a) for a in (ids, seg, mask, word, pos, typ, g, b)]
     pb.check(pb.lib.cubert_op_embed_layernorm(*[a.data_ptr() for a in args], x.data_ptr(), xb.data_ptr(),
-                                              madd.data_ptr(), B, S, H, V, 2, stream()))
+                                              madd.data_ptr(), B, S, H, V, 2, 0, stream()))
     torch.cuda.synchronize()
     got = x.cpu().numpy().reshape(B, S, H)
     assert np.abs(got - ref).max() < 2e-5
@@ -223,7 +260,7 @@ def test_embed_layernorm(pb):
     # mask == NULL: everything valid
     pb.check(pb.lib.cubert_op_embed_layernorm(args[0].data_ptr(), args[1].data_ptr(), None,
                                               *[a.data_ptr() for a in args[3:]], x.data_ptr(), None,
-                                              madd.data_ptr(), B, S, H, V, 2, stream()))
+                                              madd.data_ptr(), B, S, H, V, 2, 0, stream()))
     torch.cuda.synchronize()
     assert (madd.cpu().numpy()[:, :S] == 0).all()
 
@@ -250,3 +287,93 @@ def test_mask_softmax(pb, elt, B, R, S):
     assert np.abs(got - ref).max() < (1e-6 if elt == F32 else 4e-3)
     assert np.abs(got.sum(-1) - 1).max() < (1e-5 if elt == F32 else 2e-2)
     assert (got[np.broadcast_to(mask[:, None, :] == 0, got.shape)] == 0).all()
+
+
+@pytest.mark.parametrize("tile,flags_extra", [(64, 0), (128, 0), (256, 0), (256, 8)])
+@pytest.mark.parametrize("M,N,K,epi,xp,wp,yp", [(200, 128, 128, 0, 1, 1, 0), (333, 384, 256, 1, 1, 1, 1), (512, 1024, 1024, 0, 1, 0, 0),
+                                               (700, 512, 512, 0, 0, 1, 1), (1000, 768, 3072, 0, 1, 1, 0)])
+def test_gemm_packed_operands(pb, tile, flags_extra, M, N, K, epi, xp, wp, yp):
+    """bf16 GEMM reading packed X / W and writing a packed Y; every kernel variant."""
+    print("gemm packed", tile, flags_extra, M, N, K, epi, xp, wp, yp, flush=True)
+    rng = np.random.default_rng(M + N + K)
+    X = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    W = bf16_round((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    b = rng.standard_normal(N).astype(np.float32)
+    ref = X.astype(np.float64) @ W.astype(np.float64).T + b
+    if epi == 1:
+        ref = gelu64(ref)
+    Xd = torch.from_numpy(pack_p64(bf16_bits(X)).view(np.int16)).cuda() if xp else dev(X, torch.bfloat16)
+    Wd = torch.from_numpy(pack_p64(bf16_bits(W)).view(np.int16)).cuda() if wp else dev(W, torch.bfloat16)
+    bd = dev(b)
+    out_elt = BF16 if yp else F32
+    if yp:
+        Y = torch.zeros(pb.lib.cubert_packed_bytes(M, N * 2) // 2, dtype=torch.int16, device="cuda")
+    else:
+        Y = torch.full((M, N), float("nan"), device="cuda")
+    flags = xp * pb.X_PACKED + wp * pb.W_PACKED + yp * pb.Y_PACKED + flags_extra
+    pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), M, N, K, K, BF16,
+                                   out_elt, epi, tile, flags, stream()))
+    torch.cuda.synchronize()
+    if yp:
+        got = bits_to_f32(Y.cpu().numpy().view(np.uint16)[packed_index(M, N)]).astype(np.float64)
+        tol = 2e-2 * max(1.0, np.abs(ref).max() / 4)
+    else:
+        got = Y.cpu().numpy().astype(np.float64)
+        tol = 2e-4
+    assert np.isfinite(got).all()
+    assert np.abs(got - ref).max() < tol, np.abs(got - ref).max()
+
+
+def test_packed_producers(pb):
+    """LayerNorm, embedding and attention writing their bf16 result packed."""
+    rng = np.random.default_rng(3)
+    rows, H = 600, 768
+    x = rng.standard_normal((rows, H)).astype(np.float32)
+    y = rng.standard_normal((rows, H)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(H)).astype(np.float32)
+    xd, yd, gd, bd = dev(x), dev(y), dev(g), dev(b)
+    xb = torch.zeros(pb.lib.cubert_packed_bytes(rows, H * 2) // 2, dtype=torch.int16, device="cuda")
+    pb.check(pb.lib.cubert_op_add_layernorm(xd.data_ptr(), yd.data_ptr(), F32, gd.data_ptr(), bd.data_ptr(),
+                                            xb.data_ptr(), rows, H, pb.Y_PACKED, stream()))
+    torch.cuda.synchronize()
+    got32 = xd.cpu().numpy()
+    assert np.array_equal(xb.cpu().numpy().view(np.uint16)[packed_index(rows, H)], bf16_bits(got32))
+    # attention with a packed context
+    B, S, heads = 3, 100, 4
+    Sp = 128
+    q = bf16_round(rng.standard_normal((B, heads, S, 64)).astype(np.float32))
+    k = bf16_round(rng.standard_normal((B, heads, S, 64)).astype(np.float32))
+    v = bf16_round(rng.standard_normal((B, heads, S, 64)).astype(np.float32))
+    vt = np.zeros((B, heads, 64, Sp), np.float32)
+    vt[..., :S] = v.transpose(0, 1, 3, 2)
+    maskadd = np.full((B, Sp), -np.inf, np.float32)
+    maskadd[:, :S] = 0
+    qd, kd, vd, md = dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(vt, torch.bfloat16), dev(maskadd)
+    plain = torch.zeros((B * S, heads * 64), dtype=torch.bfloat16, device="cuda")
+    packed = torch.zeros(pb.lib.cubert_packed_bytes(B * S, heads * 128) // 2, dtype=torch.int16, device="cuda")
+    pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), plain.data_ptr(),
+                                        B, heads, S, 0.125, BF16, 0, stream()))
+    pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), packed.data_ptr(),
+                                        B, heads, S, 0.125, BF16, pb.Y_PACKED, stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(packed.cpu().numpy().view(np.uint16)[packed_index(B * S, heads * 64)],
+                          plain.view(torch.int16).cpu().numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("w_elt", [F32, BF16])
+def test_pooler(pb, w_elt):
+    rng = np.random.default_rng(9)
+    B, S, H = 5, 7, 768
+    seq = rng.standard_normal((B, S, H)).astype(np.float32)
+    W = (rng.standard_normal((H, H)) * 0.05).astype(np.float32)
+    if w_elt == BF16:
+        W = bf16_round(W)
+    b = rng.standard_normal(H).astype(np.float32)
+    ref = np.tanh(seq[:, 0].astype(np.float64) @ W.T.astype(np.float64) + b)
+    out = torch.zeros((B, H), device="cuda")
+    xd, wd, bd = dev(seq), dev(W, torch.float32 if w_elt == F32 else torch.bfloat16), dev(b)
+    pb.check(pb.lib.cubert_op_pooler(xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), out.data_ptr(), B, S, H, w_elt,
+                                     stream()))
+    torch.cuda.synchronize()
+    assert np.abs(out.cpu().numpy() - ref).max() < 2e-5, np.abs(out.cpu().numpy() - ref).max()
