@@ -170,7 +170,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #undef CUBERT_LOAD_FRAGS
 #undef CUBERT_K_STEP
 
-    gemm_epilogue<OUT, EPI, NB>(p, acc, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g);
+    // every wave is past the last step's barrier: the tiles are dead, lds0 is free for staging
+    gemm_epilogue<OUT, EPI, NB>(p, acc, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
 }
 
 template <int ELT, int OUT, int EPI, int BT>
@@ -222,6 +223,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0 || p.K <= 0) { set_error("gemm: empty problem"); return false; }
     if (p.K % bk != 0) { set_error("gemm: K must be a multiple of " + std::to_string(bk)); return false; }
     if (p.N % 4 != 0) { set_error("gemm: N must be a multiple of 4"); return false; }
+    if (p.out_elt == kBF16 && p.N % 8 != 0) { set_error("gemm: N must be a multiple of 8 for bf16 results"); return false; }
     if (!p.x_packed && (p.ldx < p.K || (p.ldx * es) % 16 != 0)) { set_error("gemm: bad ldx"); return false; }
     if (p.x_packed && p.ldx != p.K) { set_error("gemm: a packed X has no row stride"); return false; }
     if (!p.X || !p.W || !p.bias) { set_error("gemm: null operand"); return false; }

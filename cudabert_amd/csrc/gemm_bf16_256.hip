@@ -84,7 +84,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
           CUBERT_V10(18), CUBERT_V10(19), CUBERT_V10(20), CUBERT_V10(21), CUBERT_V10(22), CUBERT_V10(23),
           CUBERT_V10(24), "v250", "v251", "v252", "v253", "v254", "v255");
 
-    gemm_epilogue<OUT, EPI, 4>(p, acc, n0 + wn * 128, m0 + wm * 128, l32, g);
+    // Stages 0 and 1 were last read two barriers ago; the tail of the loop only reads stages
+    // 2 and 3, so the first 64 KiB are free for the epilogue's staging while slower waves finish.
+    gemm_epilogue<OUT, EPI, 4>(p, acc, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
 }
 
 template <int OUT>

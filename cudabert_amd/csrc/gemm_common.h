@@ -92,13 +92,32 @@ __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, i
 // owns token column l32 of block j and, per accumulator quad qd, the four
 // consecutive feature rows 8 qd + 4 g + {0..3} of block i.  n_base / m_base are
 // the first feature / token of this wave's quadrant.
+//
+// Written straight from that layout every store instruction would touch 32
+// different output rows with 8 or 16 bytes each, and the memory pipeline takes
+// longer over those than the MFMAs took over the tile.  So each block row j
+// (32 tokens x 32 NB features) goes through a wave-private piece of LDS
+// (`scratch`, 32 * 32 NB * sizeof(out) bytes, twice that for bf16 so that
+// consecutive j alternate halves): the lanes write their quads at
+// [token][feature] with the 16-byte chunk index XORed with the token number
+// (spreads the column of writes over all banks), then read whole rows back so
+// that a store instruction covers complete 256/512-byte row segments.
+// The V part of a fused QKV projection is stored transposed ([.., 64, Sp],
+// token-contiguous), which is the accumulator's own orientation: it skips the LDS.
 template <int OUT, int EPI, int NB>
 __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NB][NB], int n_base, int m_base,
-                                              int l32, int g) {
+                                              int l32, int g, unsigned char* scratch) {
+    constexpr int OES = (OUT == kBF16) ? 2 : 4;
+    constexpr int RB = 32 * NB * OES;       // bytes per token row of the staging block
+    constexpr int CH = RB / 16;             // 16-byte chunks per row
+    constexpr int RPI = 64 / CH;            // rows one store instruction covers
+    constexpr int EPC = 16 / OES;           // elements per chunk
+    const int lane = l32 + 32 * g;
+    const int rrow = lane / CH, rc = lane % CH;
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
+        unsigned char* buf = scratch + ((OES == 2 && (j & 1)) ? 32 * RB : 0);
         const int m = m_base + 32 * j + l32;
-        if (m >= p.M) continue;
         int bidx = 0, sidx = 0;
         if constexpr (EPI == kEpiQKV) {
             bidx = m / p.S;
@@ -108,7 +127,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
         for (int i = 0; i < NB; ++i) {
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
-                const int n = n_base + 32 * i + 8 * qd + 4 * g;
+                const int fq = 32 * i + 8 * qd + 4 * g;          // feature within the quadrant
+                const int n = n_base + fq;
                 if (n >= p.N) continue;
                 const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(p.bias + n);
                 float v[4];
@@ -120,24 +140,40 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                     v[e] = t;
                 }
                 if constexpr (EPI == kEpiQKV) {
-                    const int which = n / p.hidden;
-                    const int hn = n - which * p.hidden;
-                    const int head = hn >> 6, dd = hn & 63;
-                    const size_t bh = (size_t)bidx * p.heads + head;
-                    if (which == 2) {
-                        const size_t base = (bh * 64 + dd) * p.Sp + sidx;
+                    if (n >= 2 * p.hidden) {
+                        if (m < p.M) {
+                            const int hn = n - 2 * p.hidden;
+                            const size_t bh = (size_t)bidx * p.heads + (hn >> 6);
+                            const size_t base = (bh * 64 + (hn & 63)) * p.Sp + sidx;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) store1<OUT>(p.vt, base + (size_t)e * p.Sp, v[e]);
-                    } else {
-                        store4<OUT>(which == 0 ? p.q : p.k, (bh * p.S + sidx) * 64 + dd, v);
+                            for (int e = 0; e < 4; ++e) store1<OUT>(p.vt, base + (size_t)e * p.Sp, v[e]);
+                        }
+                        continue;
                     }
-                } else if (p.y_packed) {
-                    // packed bf16 result: the next GEMM's activation operand
-                    bf16x4_t o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-                    *reinterpret_cast<bf16x4_t*>(p.Y + packed_offset(m, n * 2, p.N * 2 / 64)) = o;
-                } else {
-                    store4<OUT>(p.Y, (size_t)m * p.N + n, v);
                 }
+                const int fb = fq * OES;
+                store4<OUT>(buf + l32 * RB + ((((fb >> 4) ^ l32) & (CH - 1)) << 4) + (fb & 15), 0, v);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 32 / RPI; ++s) {
+            const int row = s * RPI + rrow;
+            const u32x4_t d = *reinterpret_cast<const u32x4_t*>(buf + row * RB + (((rc ^ row) & (CH - 1)) << 4));
+            const int mm = m_base + 32 * j + row;
+            const int n = n_base + rc * EPC;
+            if (mm >= p.M || n >= p.N) continue;
+            if constexpr (EPI == kEpiQKV) {
+                if (n >= 2 * p.hidden) continue;
+                const int b2 = mm / p.S, s2 = mm - b2 * p.S;
+                const int which = n >= p.hidden ? 1 : 0;
+                const int hn = n - which * p.hidden;
+                const size_t bh = (size_t)b2 * p.heads + (hn >> 6);
+                *reinterpret_cast<u32x4_t*>((which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES) = d;
+            } else if (p.y_packed) {
+                // packed bf16 result: the next GEMM's activation operand
+                *reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)) = d;
+            } else {
+                *reinterpret_cast<u32x4_t*>(p.Y + ((size_t)mm * p.N + n) * OES) = d;
             }
         }
     }
