@@ -170,8 +170,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #undef CUBERT_LOAD_FRAGS
 #undef CUBERT_K_STEP
 
+    f32x4_t bias[4 * NB];      // fetched here rather than before the loop: no registers to spare there
+    gemm_load_bias<NB>(p, n0 + wn * (BT / 2), g, bias);
     // every wave is past the last step's barrier: the tiles are dead, lds0 is free for staging
-    gemm_epilogue<OUT, EPI, NB>(p, acc, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
+    gemm_epilogue<OUT, EPI, NB>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
 }
 
 template <int ELT, int OUT, int EPI, int BT>

@@ -72,6 +72,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     const int ht = p.K / 32;          // half-steps; a multiple of 4
 
     f32x16_t acc[4][4];       // zeroed inside the asm block
+    f32x4_t bias[16];
+    gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
 
     asm volatile(
 #include "gemm_bf16_256_loop.inc"
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
 
     // Stages 0 and 1 were last read two barriers ago; the tail of the loop only reads stages
     // 2 and 3, so the first 64 KiB are free for the epilogue's staging while slower waves finish.
-    gemm_epilogue<OUT, EPI, 4>(p, acc, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
+    gemm_epilogue<OUT, EPI, 4>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
 }
 
 template <int OUT>
