@@ -52,6 +52,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.dims.inter = cfg.intermediate;
     opt.precision = cfg.precision;
     opt.graph_max_tokens = cfg.graph_max_tokens;
+    opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;

@@ -45,6 +45,9 @@ Model::~Model() {
     if (wblock_) (void)hipFree(wblock_);
     if (ablock_) (void)hipFree(ablock_);
     if (h_in_) (void)hipHostFree(h_in_);
+    if (ev_fork_) (void)hipEventDestroy(ev_fork_);
+    if (ev_join_) (void)hipEventDestroy(ev_join_);
+    if (stream2_) (void)hipStreamDestroy(stream2_);
     if (stream_) (void)hipStreamDestroy(stream_);
 }
 
@@ -83,6 +86,9 @@ bool Model::init(const ModelOptions& opt_in) {
     }
     CUBERT_HIP_OK(hipSetDevice(opt_.gpu));
     CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+    CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream2_, hipStreamNonBlocking));
+    CUBERT_HIP_OK(hipEventCreateWithFlags(&ev_fork_, hipEventDisableTiming));
+    CUBERT_HIP_OK(hipEventCreateWithFlags(&ev_join_, hipEventDisableTiming));
 
     const int elt = opt_.precision;
     const size_t es = elt == kBF16 ? 2 : 4;
@@ -170,7 +176,8 @@ bool Model::init(const ModelOptions& opt_in) {
 
     // ---- activation block: one allocation, addresses fixed for the model's life ----
     // B <= 1024 and every sequence is padded by < 32 key columns in vt/maskadd.
-    const size_t N = ((size_t)cap_tokens_ + 255) / 256 * 256;     // packed operands pad rows to 256
+    // Packed operands pad rows to 256; a batch split over the two streams has two such regions.
+    const size_t N = ((size_t)cap_tokens_ + 255) / 256 * 256 + 256;
     const size_t Npad = N + 32 * 1024;
     Arena aa;
     const size_t o_x32 = aa.take(N * H * 4);
@@ -287,21 +294,53 @@ bool Model::run(int B, int S, bool has_mask) {
     return true;
 }
 
-// The launch sequence of one forward pass (cuda_bert/utils/bert.cu:129-252):
-// 1 + 7 * layers + 1 kernels, no host synchronisation.
+// One forward pass.  A large batch is cut into two halves of whole sequences that
+// run the same launch sequence on two streams: the halves are independent, and
+// while one half's GEMM is in its last, partly filled round of tiles (or in a
+// bandwidth-bound row kernel) the other half's kernel takes the idle CUs.
 bool Model::enqueue(int B, int S, bool has_mask) {
+    const long tokens = (long)B * S;
+    if (profiling_ || B < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens)
+        return enqueue_part(0, B, 0, S, has_mask, stream_);
+    const int B0 = (B + 1) / 2;
+    CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
+    CUBERT_HIP_OK(hipStreamWaitEvent(stream2_, ev_fork_, 0));
+    const bool ok = enqueue_part(0, B0, 0, S, has_mask, stream_) &&
+                    enqueue_part(B0, B - B0, (size_t)round_up(B0 * S, 256), S, has_mask, stream2_);
+    // join even after a failed launch so that a capture in progress can be closed
+    CUBERT_HIP_OK(hipEventRecord(ev_join_, stream2_));
+    CUBERT_HIP_OK(hipStreamWaitEvent(stream_, ev_join_, 0));
+    return ok;
+}
+
+// The launch sequence for sequences [b0, b0 + B) (cuda_bert/utils/bert.cu:129-252):
+// 1 + 7 * layers + 1 kernels, no host synchronisation.  `r0` is the first row of
+// this part in the internal activation buffers (a multiple of 256, so that a
+// packed operand starts on a block boundary); inputs and the sequence output
+// are indexed by token.
+bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st) {
     const Dims& D = opt_.dims;
     const int elt = opt_.precision;
+    const size_t es = elt == kBF16 ? 2 : 4;
     const int H = D.hidden, I = D.inter, N = B * S, Sp = round_up(S, 32);
-    const size_t cap = (size_t)cap_tokens_;
-    const int *ids = d_in_, *seg = d_in_ + cap, *mask = has_mask ? d_in_ + 2 * cap : nullptr;
-    const void* xin = elt == kBF16 ? static_cast<const void*>(xb_) : static_cast<const void*>(x32_);
+    const size_t cap = (size_t)cap_tokens_, t0 = (size_t)b0 * S;
+    const int *ids = d_in_ + t0, *seg = d_in_ + cap + t0, *mask = has_mask ? d_in_ + 2 * cap + t0 : nullptr;
+    float* x32 = x32_ + t0 * H;
+    float* y32 = y32_ + r0 * H;
+    bf16_t* xb = xb_ ? xb_ + r0 * H : nullptr;
+    unsigned char* q = static_cast<unsigned char*>(q_) + t0 * H * es;
+    unsigned char* k = static_cast<unsigned char*>(k_) + t0 * H * es;
+    unsigned char* vt = static_cast<unsigned char*>(vt_) + (size_t)b0 * H * Sp * es;
+    unsigned char* ctx = static_cast<unsigned char*>(ctx_) + r0 * H * es;
+    unsigned char* h = static_cast<unsigned char*>(h_) + r0 * I * es;
+    float* maskadd = maskadd_ + (size_t)b0 * Sp;
+    const void* xin = elt == kBF16 ? static_cast<const void*>(xb) : static_cast<const void*>(x32);
     const float scale = 1.0f / std::sqrt(64.0f);
 
     if (!mark(kPhEmbed)) return false;
     const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
-    if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32_, xb_, pk, maskadd_, B, S, Sp,
-                                H, D.vocab, D.type_vocab, stream_))
+    if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32, xb, pk, maskadd, B, S, Sp,
+                                H, D.vocab, D.type_vocab, st))
         return false;
     for (int i = 0; i < D.layers; ++i) {
         const LayerDev& L = layers_[i];
@@ -309,33 +348,33 @@ bool Model::enqueue(int B, int S, bool has_mask) {
         g.elt = elt;
         // QKV projection, scattered per head (V transposed)
         g.X = xin; g.ldx = H; g.W = L.w_qkv; g.bias = L.b_qkv; g.M = N; g.N = 3 * H; g.K = H;
-        g.epilogue = kEpiQKV; g.q = q_; g.k = k_; g.vt = vt_; g.S = S; g.Sp = Sp; g.heads = D.heads;
+        g.epilogue = kEpiQKV; g.q = q; g.k = k; g.vt = vt; g.S = S; g.Sp = Sp; g.heads = D.heads;
         g.x_packed = g.w_packed = pk;
-        if (!mark(kPhQKV) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhQKV) || !launch_gemm(g, st)) return false;
         if (!mark(kPhAttention)) return false;
-        if (!launch_attention(q_, k_, vt_, maskadd_, ctx_, pk, B, D.heads, S, Sp, scale, elt, stream_)) return false;
+        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
-        g.elt = elt; g.out_elt = kF32; g.X = ctx_; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32_;
+        g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;
         g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
-        if (!mark(kPhAttnOut) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhAttnOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32_, y32_, kF32, L.g1, L.be1, xb_, pk, N, H, stream_)) return false;
+        if (!launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st)) return false;
         // feed-forward
         g = GemmParams();
-        g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h_;
+        g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h;
         g.M = N; g.N = I; g.K = H; g.epilogue = kEpiBiasGelu; g.x_packed = g.w_packed = g.y_packed = pk;
-        if (!mark(kPhFFNIn) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhFFNIn) || !launch_gemm(g, st)) return false;
         g = GemmParams();
-        g.elt = elt; g.out_elt = kF32; g.X = h_; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32_;
+        g.elt = elt; g.out_elt = kF32; g.X = h; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32;
         g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
-        if (!mark(kPhFFNOut) || !launch_gemm(g, stream_)) return false;
+        if (!mark(kPhFFNOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32_, y32_, kF32, L.g2, L.be2, xb_, pk, N, H, stream_)) return false;
+        if (!launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st)) return false;
     }
     // pooler: first-token gather + dense + tanh on the float32 sequence output
     if (!mark(kPhPooler)) return false;
-    return launch_pooler(x32_, w_pool_, elt, b_pool_, pooled_, B, S, H, stream_);
+    return launch_pooler(x32, w_pool_, elt, b_pool_, pooled_ + (size_t)b0 * H, B, S, H, st);
 }
 
 bool Model::mark(int phase) {

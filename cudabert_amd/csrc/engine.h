@@ -22,6 +22,7 @@ struct ModelOptions {
     int gpu = 0;
     int max_batch = 0;         // (0, 0): default capacity of 200*512 tokens
     int max_seq = 0;
+    int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
     std::string dir;
 };
@@ -72,11 +73,14 @@ class Model {
     bool init(const ModelOptions& opt);
     bool check_shape(int B, int S);
     bool run(int B, int S, bool has_mask);             // graph or eager
-    bool enqueue(int B, int S, bool has_mask);         // the launch sequence
+    bool enqueue(int B, int S, bool has_mask);         // the launch sequence (one or two parts)
+    bool enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st);
     bool mark(int phase);                              // profiling: event before a launch
 
     ModelOptions opt_;
     hipStream_t stream_ = nullptr;
+    hipStream_t stream2_ = nullptr;              // second half of a split batch
+    hipEvent_t ev_fork_ = nullptr, ev_join_ = nullptr;
     // weights
     unsigned char* wblock_ = nullptr;
     size_t weight_bytes_ = 0;

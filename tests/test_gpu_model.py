@@ -223,3 +223,34 @@ def test_padding_and_permutation_properties(pb, base_dir):
     assert np.abs(pooled2 - pooled).max() < 2e-3
     assert np.array_equal(seq3, seq[perm]) and np.array_equal(pooled3, pooled[perm])
     assert np.isfinite(seq).all() and np.abs(pooled).max() < 1.0
+
+
+@pytest.mark.parametrize("precision", [F32, BF16])
+def test_split_batch_two_streams_is_bit_identical(pb, tiny_dir, precision, monkeypatch):
+    """A batch cut into two halves on two streams (what large batches get) must give
+    exactly the bits of the single-stream pass: every output row depends only on its
+    own sequence.  Odd batch, ragged lengths, eager and graph replay."""
+    wdir = str(tiny_dir / ("f32" if precision == F32 else "bf16"))
+    npy = W.load_npy_dir(wdir)
+    B, S = 5, 37
+    ids, seg, mask = synth.make_inputs(B, S, [37, 3, 20, 1, 29], vocab=W.TINY.vocab, seed=99, prune=False)
+    monkeypatch.setenv("CUBERT_SPLIT_MIN_TOKENS", "0")
+    whole = load(pb, W.TINY, wdir, precision, B, S)
+    monkeypatch.setenv("CUBERT_SPLIT_MIN_TOKENS", "1")
+    split = load(pb, W.TINY, wdir, precision, B, S)
+    split_graph = load(pb, W.TINY, wdir, precision, B, S, graph=4096)
+    try:
+        pooled0, seq0, cls0 = pb.encode(whole, ids, seg, mask, want_seq=True)
+        seq_ref, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+        assert np.abs(seq0 - seq_ref).max() < TOL[precision]
+        for m, reps in ((split, 2), (split_graph, 4)):
+            for _ in range(reps):
+                pooled1, seq1, cls1 = pb.encode(m, ids, seg, mask, want_seq=True)
+                assert np.array_equal(seq0, seq1)
+                assert np.array_equal(pooled0, pooled1)
+                if cls0 is not None:
+                    assert np.array_equal(cls0, cls1)
+        assert pb.lib.cubert_graphs_cached(split_graph) == 1
+    finally:
+        for m in (whole, split, split_graph):
+            pb.unload_model(m)
