@@ -171,6 +171,167 @@ __global__ __launch_bounds__(256) void attention_kernel(
         }
 }
 
+
+// ---------------------------------------------------------------------------
+// bf16, S <= 512: one workgroup per (batch, head) with one wave per block of 32
+// queries.  K [S, 64] and V^T [64, Sp] of the head are brought into LDS once
+// (instead of once per wave through the vector memory path) and every wave
+// takes its MFMA operands from there:
+//   K    rows of 128 bytes, 16-byte chunk c of row r in slot c ^ (r & 7)
+//        (the 32 lanes of a fragment read hit 8 different slots);
+//   V^T  rows `vstride` = 8 (mod 256) bytes apart, so that the 32 rows a
+//        fragment read touches start in 32 different bank pairs;
+//   the additive mask row, premultiplied by log2(e): the softmax runs in the
+//        exp2 domain, s' = score * (scale * log2 e) + mask * log2 e.
+// Key blocks in which every key is masked are skipped: with at least one
+// visible key in the row their probabilities are exactly zero in float32
+// (exp2 of less than -14000), so the result is bit-identical to walking them.
+// If no key at all is visible nothing is skipped.
+__global__ __launch_bounds__(1024) void attention_lds_kernel(
+    const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
+    const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
+    unsigned char* __restrict__ ctx, int heads, int S, int Sp, int vstride, float scale_log2e, int ctx_packed) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* sK = smem;
+    unsigned char* sV = smem + (size_t)Sp * 128;
+    float* sM = reinterpret_cast<float*>(sV + 64 * (size_t)vstride);
+    int* sLive = reinterpret_cast<int*>(sM + Sp);
+
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g = lane >> 5;
+    const int nblk = Sp >> 5;                  // == number of waves
+    const int h = blockIdx.x, b = blockIdx.y;
+    const size_t bh = (size_t)b * heads + h;
+    const unsigned char* qb = q + bh * S * 128;
+    const unsigned char* kb = k + bh * S * 128;
+    const unsigned char* vb = vt + bh * 64 * (size_t)Sp * 2;
+
+    // ---- stage K (rows S..Sp-1 zero), V^T and the mask row ----
+    for (int c = tid; c < Sp * 8; c += nthr) {
+        const int row = c >> 3, ch = c & 7;
+        uint4 d = {0u, 0u, 0u, 0u};
+        if (row < S) d = *reinterpret_cast<const uint4*>(kb + (size_t)c * 16);
+        *reinterpret_cast<uint4*>(sK + row * 128 + ((ch ^ (row & 7)) << 4)) = d;
+    }
+    const int vchunks = Sp >> 3;               // 16-byte chunks per V^T row
+    for (int c = tid; c < 64 * vchunks; c += nthr) {
+        const int row = c / vchunks, ch = c - row * vchunks;
+        const uint4 d = *reinterpret_cast<const uint4*>(vb + ((size_t)row * Sp + ch * 8) * 2);
+        uint2* dst = reinterpret_cast<uint2*>(sV + (size_t)row * vstride + ch * 16);     // rows are 8-byte aligned
+        dst[0] = make_uint2(d.x, d.y);
+        dst[1] = make_uint2(d.z, d.w);
+    }
+    {
+        // wave w looks at mask block w
+        const float m = lane < 32 ? maskadd[(size_t)b * Sp + wave * 32 + lane] : -INFINITY;
+        if (lane < 32) sM[wave * 32 + lane] = m * 1.4426950408889634f;
+        const unsigned long long vis = __ballot(m > -5000.0f);
+        if (lane == 0) sLive[wave] = vis != 0ull ? 1 : 0;
+    }
+    __syncthreads();
+    unsigned live = 0;
+    for (int i = 0; i < nblk; ++i) live |= sLive[i] ? (1u << i) : 0u;
+    if (live == 0) live = 0xffffffffu;
+    live = __builtin_amdgcn_readfirstlane(live);
+
+    // Q fragments ("B" operand: column = query), kept for the whole key loop.
+    const int q0 = wave * 32;
+    int qrow = q0 + l32;
+    qrow = qrow < S ? qrow : S - 1;
+    uint4 qf[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+        qf[kk] = *reinterpret_cast<const uint4*>(qb + (size_t)qrow * 128 + (2 * kk + g) * 16);
+
+    f32x16_t o[2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
+    float run_max = -INFINITY, run_sum = 0.0f;
+    const int ksw = l32 & 7;
+
+    for (int kblk = 0; kblk < nblk; ++kblk) {
+        if (!((live >> kblk) & 1u)) continue;
+        const int k0 = kblk * 32;
+        // ---- scores^T block: rows = keys k0..k0+31, column = my query ----
+        f32x16_t sc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] = 0.0f;
+        const unsigned char* krow = sK + (k0 + l32) * 128;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const uint4 kf = *reinterpret_cast<const uint4*>(krow + (((2 * kk + g) ^ ksw) << 4));
+            sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf),
+                                                         __builtin_bit_cast(bf16x8_t, qf[kk]), sc, 0, 0, 0);
+        }
+        float blk_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f32x4_t m4 = *reinterpret_cast<const f32x4_t*>(sM + k0 + 8 * j + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float t = fmaf(sc[4 * j + e], scale_log2e, m4[e]);
+                sc[4 * j + e] = t;
+                blk_max = fmaxf(blk_max, t);
+            }
+        }
+        blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+        const float new_max = fmaxf(run_max, blk_max);    // finite: a processed block holds a real key column
+        const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);
+        float blk_sum = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float pv = __builtin_amdgcn_exp2f(sc[v] - new_max);
+            sc[v] = pv;
+            blk_sum += pv;
+        }
+        blk_sum += __shfl_xor(blk_sum, 32);
+        run_sum = run_sum * alpha + blk_sum;
+        run_max = new_max;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+
+        // ---- ctx^T += V^T (rows = head features) x P^T (column = my query) ----
+#pragma unroll
+        for (int f = 0; f < 2; ++f) {        // keys k0 + 16 f + {4g..4g+3, 8+4g..8+4g+3}
+            bf16x8_t pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = (__bf16)sc[8 * f + e];
+#pragma unroll
+            for (int db = 0; db < 2; ++db) {
+                const unsigned char* vrow = sV + (size_t)(32 * db + l32) * vstride + (k0 + 16 * f + 4 * g) * 2;
+                const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                const uint4 vf = {lo.x, lo.y, hi.x, hi.y};
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf), pf, o[db], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- normalise and store: lane owns query q0 + l32, features 32 db + 8 j + 4 g + e ----
+    const int qi = q0 + l32;
+    if (qi >= S) return;
+    const float inv = 1.0f / run_sum;
+    const size_t hidden = (size_t)heads * 64;
+    unsigned char* orow = ctx + (((size_t)b * S + qi) * hidden + (size_t)h * 64) * 2;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = 32 * db + 8 * j + 4 * g;
+            bf16x4_t w = {(__bf16)(o[db][4 * j] * inv), (__bf16)(o[db][4 * j + 1] * inv),
+                          (__bf16)(o[db][4 * j + 2] * inv), (__bf16)(o[db][4 * j + 3] * inv)};
+            if (ctx_packed)
+                *reinterpret_cast<bf16x4_t*>(ctx + packed_offset(b * S + qi, (h * 64 + d) * 2, (int)hidden * 2 / 64)) = w;
+            else
+                *reinterpret_cast<bf16x4_t*>(orow + d * 2) = w;
+        }
+}
+
 }  // namespace
 
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
@@ -190,11 +351,28 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
         set_error("attention: operands must be 16-byte aligned");
         return false;
     }
-    dim3 grid((S + 127) / 128, heads, B), block(256);
     const unsigned char* qc = static_cast<const unsigned char*>(q);
     const unsigned char* kc = static_cast<const unsigned char*>(k);
     const unsigned char* vc = static_cast<const unsigned char*>(vt);
     unsigned char* cc = static_cast<unsigned char*>(ctx);
+    if (elt == kBF16 && S <= 512) {
+        const int vstride = round_up(Sp * 2, 256) + 8;
+        const size_t lds = (size_t)Sp * 128 + 64 * (size_t)vstride + (size_t)Sp * 4 + 64;
+        // More than 64 KiB of dynamic LDS has to be allowed once per device.
+        static bool allowed[64] = {};
+        int dev = 0;
+        CUBERT_HIP_OK(hipGetDevice(&dev));
+        if (dev < 0 || dev >= 64 || !allowed[dev]) {
+            CUBERT_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_lds_kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            if (dev >= 0 && dev < 64) allowed[dev] = true;
+        }
+        hipLaunchKernelGGL(attention_lds_kernel, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd, cc,
+                           heads, S, Sp, vstride, scale * 1.4426950408889634f, cp);
+        CUBERT_HIP_OK(hipGetLastError());
+        return true;
+    }
+    dim3 grid((S + 127) / 128, heads, B), block(256);
     if (elt == kBF16)
         hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp);
     else

@@ -177,7 +177,13 @@ def test_attention(pb, elt, B, S, heads):
     v = rng.standard_normal((B, heads, S, 64)).astype(np.float32)
     lens = rng.integers(1, S + 1, size=B)
     lens[0] = S
+    if B >= 3:
+        lens[1] = 0            # nothing visible: every key gets -10000, i.e. an unmasked softmax
     mask = (np.arange(S)[None, :] < lens[:, None]).astype(np.float32)
+    if B >= 4:                 # a mask that is not a prefix: holes, and whole 32-key blocks masked in the middle
+        mask[2] = (rng.random(S) < 0.5).astype(np.float32)
+        mask[2, 32:96] = 0
+        mask[2, 0] = 1
     tdt = torch.float32 if elt == F32 else torch.bfloat16
     if elt == BF16:
         q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
