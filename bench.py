@@ -30,6 +30,46 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 PEAK_HBM_GBS = 8000.0
 
 
+def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
+    # ---- roofline of the dominant kernel: the FFN-in GEMM (bias+GELU epilogue) ----
+    # Same launch as in the model: in bf16 mode all three matrices are in the packed
+    # operand layout (their contents are random, only the layout matters for timing).
+    tdt = torch.bfloat16 if prec == pybert.BF16 else torch.float32
+    packed = prec == pybert.BF16
+    rows_x = (N + 255) // 256 * 256 if packed else N
+    rows_w = (I + 255) // 256 * 256 if packed else I
+    X = (torch.randn((rows_x, H), device="cuda") * 1.0).to(tdt)
+    Wt = (torch.randn((rows_w, H), device="cuda") * 0.02).to(tdt)
+    bias = torch.zeros(I, device="cuda")
+    Y = torch.empty((rows_x, I), dtype=tdt, device="cuda")
+    st = torch.cuda.current_stream()
+    out_elt = prec
+    gflags = (pybert.X_PACKED | pybert.W_PACKED | pybert.Y_PACKED) if packed else 0
+
+    def ffn_in():
+        pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H, prec,
+                                        out_elt, 1, 0, gflags, st.cuda_stream))
+    for _ in range(3):
+        ffn_in()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    launches = 20
+    e0.record(st)
+    for _ in range(launches):
+        ffn_in()
+    e1.record(st)
+    e1.synchronize()
+    k_ms = e0.elapsed_time(e1) / launches
+    flops_per_launch = 2.0 * N * H * I
+    achieved = flops_per_launch / k_ms / 1e9
+    roofline = {"bound": "mfma", "kernel": "gemm_kernel<%s, bias+GELU, tile 256> (FFN-in %dx%dx%d)" %
+                (precision, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[precision],
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[precision], 4),
+                "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch, "traffic": None}
+    del X, Wt, Y
+    return roofline
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -39,6 +79,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 4])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seqs", type=int, default=128, help="sequences in the CPU baseline sample")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="only the dominant kernel's launches plus one device copy of known size "
+                         "(the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters); for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU; --gpus %d is not supported (every replica of the "
@@ -62,6 +105,17 @@ def main():
     N = B * S
     H, I, L, A = dims.hidden, dims.inter, dims.layers, dims.heads
     es = 2 if prec == pybert.BF16 else 4
+
+    if args.roofline_only:
+        lib = pybert.lib
+        roofline = roofline_leg(torch, pybert, lib, prec, args.precision, N, I, H)
+        a = torch.empty(64 << 20, dtype=torch.float32, device="cuda")     # 256 MiB read + 256 MiB written
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"roofline": roofline, "calibration_copy_bytes_each_way": a.numel() * 4}))
+        return
 
     t0 = time.time()
     state = W.synth_state(dims, seed=20240, degenerate=True)
@@ -130,41 +184,7 @@ def main():
     phases["all_gemms"] = {"ms": round(float(gemm_ms), 3), "tflops": round(gemm_flops / gemm_ms / 1e9, 1),
                            "frac_mfma_peak": round(gemm_flops / gemm_ms / 1e9 / PEAK_TFLOPS[args.precision], 4)}
 
-    # ---- roofline of the dominant kernel: the FFN-in GEMM (bias+GELU epilogue) ----
-    # Same launch as in the model: in bf16 mode all three matrices are in the packed
-    # operand layout (their contents are random, only the layout matters for timing).
-    tdt = torch.bfloat16 if prec == pybert.BF16 else torch.float32
-    packed = prec == pybert.BF16
-    rows_x = (N + 255) // 256 * 256 if packed else N
-    rows_w = (I + 255) // 256 * 256 if packed else I
-    X = (torch.randn((rows_x, H), device="cuda") * 1.0).to(tdt)
-    Wt = (torch.randn((rows_w, H), device="cuda") * 0.02).to(tdt)
-    bias = torch.zeros(I, device="cuda")
-    Y = torch.empty((rows_x, I), dtype=tdt, device="cuda")
-    st = torch.cuda.current_stream()
-    out_elt = prec
-    gflags = (pybert.X_PACKED | pybert.W_PACKED | pybert.Y_PACKED) if packed else 0
-
-    def ffn_in():
-        pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H, prec,
-                                        out_elt, 1, 0, gflags, st.cuda_stream))
-    for _ in range(3):
-        ffn_in()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    launches = 20
-    e0.record(st)
-    for _ in range(launches):
-        ffn_in()
-    e1.record(st)
-    e1.synchronize()
-    k_ms = e0.elapsed_time(e1) / launches
-    flops_per_launch = 2.0 * N * H * I
-    achieved = flops_per_launch / k_ms / 1e9
-    roofline = {"bound": "mfma", "kernel": "gemm_kernel<%s, bias+GELU, tile 256> (FFN-in %dx%dx%d)" %
-                (args.precision, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[args.precision],
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[args.precision], 4),
-                "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch, "traffic": None}
-    del X, Wt, Y
+    roofline = roofline_leg(torch, pybert, lib, prec, args.precision, N, I, H)
 
     # ---- CPU baseline: the oracle on a bounded sample of the same batch ----
     cpu = None

@@ -53,6 +53,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.precision = cfg.precision;
     opt.graph_max_tokens = cfg.graph_max_tokens;
     opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
+    opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;

@@ -46,8 +46,10 @@ Model::~Model() {
     if (ablock_) (void)hipFree(ablock_);
     if (h_in_) (void)hipHostFree(h_in_);
     if (ev_fork_) (void)hipEventDestroy(ev_fork_);
-    if (ev_join_) (void)hipEventDestroy(ev_join_);
-    if (stream2_) (void)hipStreamDestroy(stream2_);
+    for (int i = 1; i < kMaxParts; ++i) {
+        if (ev_join_[i]) (void)hipEventDestroy(ev_join_[i]);
+        if (side_[i]) (void)hipStreamDestroy(side_[i]);
+    }
     if (stream_) (void)hipStreamDestroy(stream_);
 }
 
@@ -86,9 +88,11 @@ bool Model::init(const ModelOptions& opt_in) {
     }
     CUBERT_HIP_OK(hipSetDevice(opt_.gpu));
     CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
-    CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream2_, hipStreamNonBlocking));
+    for (int i = 1; i < kMaxParts; ++i) {
+        CUBERT_HIP_OK(hipStreamCreateWithFlags(&side_[i], hipStreamNonBlocking));
+        CUBERT_HIP_OK(hipEventCreateWithFlags(&ev_join_[i], hipEventDisableTiming));
+    }
     CUBERT_HIP_OK(hipEventCreateWithFlags(&ev_fork_, hipEventDisableTiming));
-    CUBERT_HIP_OK(hipEventCreateWithFlags(&ev_join_, hipEventDisableTiming));
 
     const int elt = opt_.precision;
     const size_t es = elt == kBF16 ? 2 : 4;
@@ -176,8 +180,8 @@ bool Model::init(const ModelOptions& opt_in) {
 
     // ---- activation block: one allocation, addresses fixed for the model's life ----
     // B <= 1024 and every sequence is padded by < 32 key columns in vt/maskadd.
-    // Packed operands pad rows to 256; a batch split over the two streams has two such regions.
-    const size_t N = ((size_t)cap_tokens_ + 255) / 256 * 256 + 256;
+    // Packed operands pad rows to 256; a batch split over several streams has one such region per part.
+    const size_t N = ((size_t)cap_tokens_ + 255) / 256 * 256 + 256 * (kMaxParts - 1);
     const size_t Npad = N + 32 * 1024;
     Arena aa;
     const size_t o_x32 = aa.take(N * H * 4);
@@ -294,22 +298,32 @@ bool Model::run(int B, int S, bool has_mask) {
     return true;
 }
 
-// One forward pass.  A large batch is cut into two halves of whole sequences that
-// run the same launch sequence on two streams: the halves are independent, and
-// while one half's GEMM is in its last, partly filled round of tiles (or in a
-// bandwidth-bound row kernel) the other half's kernel takes the idle CUs.
+// One forward pass.  A large batch is cut into parts of whole sequences that run
+// the same launch sequence on separate streams: the parts are independent, and
+// while one part's GEMM is in its last, partly filled round of tiles (or in a
+// bandwidth-bound row kernel) another part's kernel takes the idle CUs.
 bool Model::enqueue(int B, int S, bool has_mask) {
     const long tokens = (long)B * S;
-    if (profiling_ || B < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens)
+    int parts = opt_.split_parts < kMaxParts ? opt_.split_parts : kMaxParts;
+    if (parts > B) parts = B;
+    if (profiling_ || parts < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens)
         return enqueue_part(0, B, 0, S, has_mask, stream_);
-    const int B0 = (B + 1) / 2;
     CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
-    CUBERT_HIP_OK(hipStreamWaitEvent(stream2_, ev_fork_, 0));
-    const bool ok = enqueue_part(0, B0, 0, S, has_mask, stream_) &&
-                    enqueue_part(B0, B - B0, (size_t)round_up(B0 * S, 256), S, has_mask, stream2_);
-    // join even after a failed launch so that a capture in progress can be closed
-    CUBERT_HIP_OK(hipEventRecord(ev_join_, stream2_));
-    CUBERT_HIP_OK(hipStreamWaitEvent(stream_, ev_join_, 0));
+    bool ok = true;
+    size_t r0 = 0;
+    for (int i = 0, b0 = 0; i < parts; ++i) {
+        const int Bi = B / parts + (i < B % parts ? 1 : 0);
+        hipStream_t st = i == 0 ? stream_ : side_[i];
+        if (i > 0) CUBERT_HIP_OK(hipStreamWaitEvent(st, ev_fork_, 0));
+        ok = ok && enqueue_part(b0, Bi, r0, S, has_mask, st);
+        // join even after a failed launch so that a capture in progress can be closed
+        if (i > 0) {
+            CUBERT_HIP_OK(hipEventRecord(ev_join_[i], st));
+            CUBERT_HIP_OK(hipStreamWaitEvent(stream_, ev_join_[i], 0));
+        }
+        b0 += Bi;
+        r0 += (size_t)round_up(Bi * S, 256);
+    }
     return ok;
 }
 

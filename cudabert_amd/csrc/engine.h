@@ -22,6 +22,7 @@ struct ModelOptions {
     int gpu = 0;
     int max_batch = 0;         // (0, 0): default capacity of 200*512 tokens
     int max_seq = 0;
+    int split_parts = 2;           // number of parts (1..4) a large batch is cut into
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
     std::string dir;
@@ -79,8 +80,9 @@ class Model {
 
     ModelOptions opt_;
     hipStream_t stream_ = nullptr;
-    hipStream_t stream2_ = nullptr;              // second half of a split batch
-    hipEvent_t ev_fork_ = nullptr, ev_join_ = nullptr;
+    static constexpr int kMaxParts = 4;
+    hipStream_t side_[kMaxParts] = {};           // streams of parts 1.. of a split batch
+    hipEvent_t ev_fork_ = nullptr, ev_join_[kMaxParts] = {};
     // weights
     unsigned char* wblock_ = nullptr;
     size_t weight_bytes_ = 0;

@@ -208,12 +208,15 @@ bool launch_epi(const GemmDev& d, int epi, int bt, hipStream_t stream) {
 
 }  // namespace
 
-int gemm_pick_tile(int M, int N) {
+int gemm_pick_tile(int M, int N, int K, int elt) {
     // Largest tile that still yields a few workgroups per CU-round; the 256
     // tile has the best MFMA:LDS ratio, the small ones fill the chip when the
-    // problem is short.
+    // problem is short.  The hand-scheduled bf16 256 kernel runs a tile at about
+    // twice the rate of the general kernel, so it is still the better choice
+    // when its tiles cover well under half of the CUs.
     auto tiles = [&](int bt) { return (long)((M + bt - 1) / bt) * ((N + bt - 1) / bt); };
     if (tiles(256) >= 256) return 256;
+    if (elt == kBF16 && K % 128 == 0 && tiles(256) >= 96) return 256;
     if (tiles(128) >= 256) return 128;
     return 64;
 }
@@ -267,7 +270,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
             return false;
         }
     }
-    const int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N);
+    const int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
     if (p.elt == kBF16) {
