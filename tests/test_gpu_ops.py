@@ -206,7 +206,11 @@ def test_attention(pb, elt, B, S, heads):
     got = ctx.float().cpu().numpy()
     assert np.isfinite(got).all()
     tol = 2e-5 * 10 if elt == F32 else 2e-2
-    assert np.abs(got - ref).max() < tol, np.abs(got - ref).max()
+    err = np.abs(got - ref).reshape(B, S, -1).max(axis=(1, 2))
+    for b in range(B):
+        # With no visible key every score sits near -10000, where float32 resolves only
+        # 1e-3: the softmax of such a row is defined to that resolution, here and in the reference.
+        assert err[b] < (5e-3 if lens[b] == 0 else tol), (b, err[b])
 
 
 @pytest.mark.parametrize("H", [128, 768, 1024])
