@@ -28,6 +28,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes of one FFN-in GEMM launch at the headline shape (bf16, packed operands),
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --roofline-only`, each
+# counter scaled by what it reads for a 256 MiB device copy (2.0 and 1.0); the summary
+# with the commands is profiles/ffn_in_gemm_cfg2_bf16_pmc.txt.
+MEASURED_TRAFFIC = {("bf16", 25600, 4096, 1024): 5.758e8}
 
 
 def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
@@ -64,10 +69,91 @@ def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
     roofline = {"bound": "mfma", "kernel": "gemm_kernel<%s, bias+GELU, tile 256> (FFN-in %dx%dx%d)" %
                 (precision, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[precision],
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[precision], 4),
-                "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch, "traffic": None}
+                "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch,
+                "traffic": MEASURED_TRAFFIC.get((precision, N, I, H))}
     del X, Wt, Y
     return roofline
 
+
+
+def latency_leg(torch, pybert, synth, model, dims, args):
+    """Config 3: BERT-large, S=200, all positions valid, batch 1 and 8; every call replays the
+    captured hipGraph of the whole forward pass.  One call = host inputs in, pooled output
+    back on the host (the reference's Cuda_Bert contract), timed with the host clock."""
+    lib = pybert.lib
+    iters = max(args.steps, 1000)
+    res = {}
+    for B in (1, 8):
+        S = 200
+        ids, seg, mask = synth.make_inputs(B, S, [S] * B, seed=20244 + B)
+        out = np.empty((B, dims.hidden), np.float32)
+        call = lambda: pybert.check(lib.cubert_encode(model, ids.ctypes.data, seg.ctypes.data, mask.ctypes.data, B, S,
+                                                      out.ctypes.data, None, None))
+        for _ in range(max(args.warmup, 5)):
+            call()
+        ts = np.empty(iters)
+        for i in range(iters):
+            t0 = time.perf_counter()
+            call()
+            ts[i] = time.perf_counter() - t0
+        res["batch%d" % B] = {"p50_ms": round(float(np.percentile(ts, 50)) * 1e3, 4),
+                              "p99_ms": round(float(np.percentile(ts, 99)) * 1e3, 4),
+                              "mean_ms": round(float(ts.mean()) * 1e3, 4), "iters": iters,
+                              "sequences_per_s": round(B / float(ts.mean()), 1)}
+    print(json.dumps({"metric": "latency per batch, BERT-large s200 on 1 MI355X (host in -> host out)", "unit": "ms",
+                      "higher_is_better": False, "n_gpus": 1, "dtype": args.precision, "data": "synthetic",
+                      "config": {"workload": "cfg3: BERT-large encoder + pooler, seq 200 all valid, hipGraph replay",
+                                 "graphs_cached": int(lib.cubert_graphs_cached(model))},
+                      "latency": res}))
+
+
+def extras_leg(torch, pybert, model, ids, seg, mask, dims, prec, steps):
+    """Host-input entry point (uploads included) and the stand-alone bandwidth-bound kernels."""
+    lib = pybert.lib
+    B, S = ids.shape
+    N, H, A = B * S, dims.hidden, dims.heads
+    out = np.empty((B, H), np.float32)
+    call = lambda: pybert.check(lib.cubert_encode(model, ids.ctypes.data, seg.ctypes.data, mask.ctypes.data, B, S,
+                                                  out.ctypes.data, None, None))
+    for _ in range(2):
+        call()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    host_rate = B * steps / (time.perf_counter() - t0)
+    st = torch.cuda.current_stream()
+
+    def timed(fn, reps=20):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(reps):
+            fn()
+        e1.record(st)
+        e1.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    ops = {}
+    x = torch.randn((N, H), device="cuda")
+    y = torch.randn((N, H), device="cuda")
+    g = torch.ones(H, device="cuda")
+    b = torch.zeros(H, device="cuda")
+    ms = timed(lambda: pybert.check(lib.cubert_op_add_layernorm(x.data_ptr(), y.data_ptr(), 0, g.data_ptr(), b.data_ptr(),
+                                                                None, N, H, 0, st.cuda_stream)))
+    by = 3.0 * N * H * 4 + 2 * H * 4
+    ops["add_layernorm_f32"] = {"ms": round(ms, 4), "bytes": by, "gbs": round(by / ms / 1e6, 1),
+                                "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    for elt, name, tdt, es in ((0, "f32", torch.float32, 4), (1, "bf16", torch.bfloat16, 2)):
+        sc = torch.randn((B, A * S, S), device="cuda").to(tdt)
+        dm = torch.from_numpy(mask).cuda()
+        ms = timed(lambda: pybert.check(lib.cubert_op_mask_softmax(sc.data_ptr(), elt, dm.data_ptr(), B, A * S, S,
+                                                                   0.125, st.cuda_stream)))
+        by = 2.0 * B * A * S * S * es + 4 * B * S
+        ops["mask_softmax_" + name] = {"ms": round(ms, 4), "bytes": by, "gbs": round(by / ms / 1e6, 1),
+                                       "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        del sc
+    return {"host_inputs_sequences_per_s": round(host_rate, 1), "ops": ops}
 
 
 def main():
@@ -76,7 +162,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--precision", choices=["bf16", "fp32"], default="bf16")
-    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 4])
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4],
+                    help="2 = headline; 3 = latency regime (B=1 and 8, hipGraph replay, p50/p99)")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the host-input entry point (PCIe inclusive) and the stand-alone "
+                         "bandwidth-bound kernels (residual+LayerNorm, scale+mask+softmax, embedding+LayerNorm)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seqs", type=int, default=128, help="sequences in the CPU baseline sample")
     ap.add_argument("--roofline-only", action="store_true",
@@ -127,9 +217,13 @@ def main():
         t_gen = time.time() - t0
         t0 = time.time()
         model = pybert.load_model_ex(wdir, H, L, A, I, precision=prec, max_batchsize=B, max_seq_length=S,
-                                     graph_max_tokens=0)
+                                     graph_max_tokens=8192 if args.config == 3 else 0)
         t_load = time.time() - t0
     lib = pybert.lib
+    if args.config == 3:
+        latency_leg(torch, pybert, synth, model, dims, args)
+        pybert.unload_model(model)
+        return
     d_ids, d_seg, d_mask = (torch.from_numpy(a).cuda() for a in (ids, seg, mask))
     torch.cuda.synchronize()
 
@@ -208,6 +302,7 @@ def main():
         pybert.check(lib.cubert_sync(model))
         assert hip.hipMemcpy(pooled.data_ptr(), lib.cubert_pooled_ptr(model), B * H * 4, 3) == 0
         cpu["pooled_max_abs_vs_gpu"] = float(np.abs(pooled.cpu().numpy()[:n] - pooled_ref).max())
+    extras = extras_leg(torch, pybert, model, ids, seg, mask, dims, prec, args.steps) if args.extras else None
     pybert.unload_model(model)
 
     out = {
@@ -224,6 +319,8 @@ def main():
         "gemm_tflop_per_step": round(gemm_flops / 1e12, 3),
         "setup_s": {"weights_generate_write": round(t_gen, 1), "model_load": round(t_load, 1)},
     }
+    if extras:
+        out["extras"] = extras
     print(json.dumps(out))
 
 

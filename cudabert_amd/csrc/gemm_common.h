@@ -91,33 +91,26 @@ __device__ __forceinline__ void store1(unsigned char* base, size_t elem_index, f
 
 // Workgroup id -> (tile_n, tile_m).  Hardware hands consecutive workgroup ids
 // to the eight XCDs round-robin; the remap gives every XCD one contiguous run
-// of the tile sequence so tiles sharing operand rows share an L2.
+// of the tile sequence so tiles sharing operand rows share an L2.  The sequence
+// itself walks groups of kGroupM tile rows column by column: the 32 tiles that
+// an XCD's CUs hold at one time then cover 4 x 8 tiles (12 operand slabs)
+// instead of 2 x 16 (18 slabs), and the next 32 reuse the same activation rows.
+constexpr int kGroupM = 4;
 __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int* tn, int* tm) {
     const int xcd = pid & 7, idx = pid >> 3;
     const int base = total >> 3, rem = total & 7;
     const int start = xcd * base + (xcd < rem ? xcd : rem);
     const int t = start + idx;
-    *tm = t / tiles_n;
-    *tn = t - *tm * tiles_n;
+    const int tiles_m = total / tiles_n;
+    const int per_group = kGroupM * tiles_n;
+    const int group = t / per_group, r = t - group * per_group;
+    const int left = tiles_m - group * kGroupM;
+    const int gm = left < kGroupM ? left : kGroupM;       // the last group may be shorter
+    const int c = r / gm;
+    *tn = c;
+    *tm = group * kGroupM + (r - c * gm);
 }
 
-
-// Epilogue.  In the 32x32 accumulator layout lane (l32 = lane % 32, g = lane / 32)
-// owns token column l32 of block j and, per accumulator quad qd, the four
-// consecutive feature rows 8 qd + 4 g + {0..3} of block i.  n_base / m_base are
-// the first feature / token of this wave's quadrant.
-//
-// Written straight from that layout every store instruction would touch 32
-// different output rows with 8 or 16 bytes each, and the memory pipeline takes
-// longer over those than the MFMAs took over the tile.  So each block row j
-// (32 tokens x 32 NB features) goes through a wave-private piece of LDS
-// (`scratch`, 32 * 32 NB * sizeof(out) bytes, twice that for bf16 so that
-// consecutive j alternate halves): the lanes write their quads at
-// [token][feature] with the 16-byte chunk index XORed with the token number
-// (spreads the column of writes over all banks), then read whole rows back so
-// that a store instruction covers complete 256/512-byte row segments.
-// The V part of a fused QKV projection is stored transposed ([.., 64, Sp],
-// token-contiguous), which is the accumulator's own orientation: it skips the LDS.
 // The bias values a lane needs (4 NB quads) are fetched by gemm_load_bias before the
 // K loop so that their latency is hidden; features past N read the last valid quad
 // (their results are never stored).
