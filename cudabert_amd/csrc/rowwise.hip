@@ -182,6 +182,121 @@ __global__ __launch_bounds__(256) void mask_softmax_kernel(unsigned char* __rest
     }
 }
 
+// Vectorised form for rows whose byte length is a multiple of 16 (S % 4 == 0 for
+// float32, S % 8 == 0 for bf16): a row is cut into 16-byte chunks, a group of LPR
+// lanes (a power of two, 8..64) owns one row and each lane U chunks, so a wave
+// moves 64/LPR whole rows with full-width loads and stores and the reductions
+// stay inside the lane group.
+template <int ELT, int U, int RU>
+__global__ __launch_bounds__(256) void mask_softmax_vec_kernel(unsigned char* __restrict__ scores,
+                                                               const int* __restrict__ mask, long rows,
+                                                               int rows_per_batch, int S, float scale, int lpr) {
+    constexpr int ES = (ELT == kBF16) ? 2 : 4;
+    constexpr int EPC = 16 / ES;                 // elements per chunk
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / lpr, sl = lane - sub * lpr;
+    // a lane group works on RU consecutive rows at a time: RU * U independent loads in flight per lane
+    const long row0 = (((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / lpr) + sub) * RU;
+    const int chunks = S / EPC;
+    uint4 raw[RU][U];
+#pragma unroll
+    for (int r = 0; r < RU; ++r)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int ci = u * lpr + sl;
+            if (row0 + r < rows && ci < chunks)
+                raw[r][u] = *reinterpret_cast<const uint4*>(scores + ((size_t)(row0 + r) * S * ES + (size_t)ci * 16));
+        }
+    // Softmax in the exp2 domain: t = s * (scale log2 e) + (1 - m) * (-10000 log2 e).  The mask
+    // terms of this lane's chunks are shared by all rows of a batch entry; they are rebuilt
+    // only when the row group crosses into the next entry.
+    const float c2 = scale * 1.4426950408889634f;
+    float madd[U][EPC];
+    int madd_b = -1;
+#pragma unroll
+    for (int r = 0; r < RU; ++r) {
+        const long row = row0 + r;
+        const bool live = row < rows;
+        const int b = live ? (int)(row / rows_per_batch) : 0;
+        if (b != madd_b) {
+            madd_b = b;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ci = u * lpr + sl;
+#pragma unroll
+                for (int e4 = 0; e4 < EPC / 4; ++e4) {
+                    int4 m4 = {1, 1, 1, 1};
+                    if (mask && ci < chunks) m4 = *reinterpret_cast<const int4*>(mask + (size_t)b * S + ci * EPC + 4 * e4);
+                    const int mm[4] = {m4.x, m4.y, m4.z, m4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) madd[u][4 * e4 + e] = (1.0f - (float)mm[e]) * -14426.950408889634f;
+                }
+            }
+        }
+        float v[U][EPC];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int ci = u * lpr + sl;
+            if (live && ci < chunks) {
+                if constexpr (ELT == kBF16) {
+                    const unsigned w[4] = {raw[r][u].x, raw[r][u].y, raw[r][u].z, raw[r][u].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[u][2 * e] = __uint_as_float(w[e] << 16);
+                        v[u][2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+                    }
+                } else {
+                    v[u][0] = __uint_as_float(raw[r][u].x); v[u][1] = __uint_as_float(raw[r][u].y);
+                    v[u][2] = __uint_as_float(raw[r][u].z); v[u][3] = __uint_as_float(raw[r][u].w);
+                }
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) {
+                    const float t = fmaf(v[u][e], c2, madd[u][e]);
+                    v[u][e] = t;
+                    mx = fmaxf(mx, t);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) v[u][e] = -INFINITY;
+            }
+        }
+        for (int m = lpr >> 1; m > 0; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
+        if (!live) mx = 0.0f;                      // keeps exp(-inf - mx) well defined for absent rows
+        float sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int e = 0; e < EPC; ++e) {
+                v[u][e] = __builtin_amdgcn_exp2f(v[u][e] - mx);     // 0 for the chunks this lane does not own
+                sum += v[u][e];
+            }
+        for (int m = lpr >> 1; m > 0; m >>= 1) sum += __shfl_xor(sum, m);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int ci = u * lpr + sl;
+            if (live && ci < chunks) {
+                uint4 o;
+                if constexpr (ELT == kBF16) {
+                    unsigned w[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const __bf16 lo = (__bf16)(v[u][2 * e] * inv), hi = (__bf16)(v[u][2 * e + 1] * inv);
+                        w[e] = (unsigned)__builtin_bit_cast(unsigned short, lo) |
+                               ((unsigned)__builtin_bit_cast(unsigned short, hi) << 16);
+                    }
+                    o = make_uint4(w[0], w[1], w[2], w[3]);
+                } else {
+                    o = make_uint4(__float_as_uint(v[u][0] * inv), __float_as_uint(v[u][1] * inv),
+                                   __float_as_uint(v[u][2] * inv), __float_as_uint(v[u][3] * inv));
+                }
+                *reinterpret_cast<uint4*>(scores + ((size_t)row * S * ES + (size_t)ci * 16)) = o;
+            }
+        }
+    }
+}
+
 // probs[b, :] = softmax(pooled[b, :] @ kernel[H, C] + bias); one wave per row.
 __global__ __launch_bounds__(64) void classifier_kernel(const float* __restrict__ pooled,
                                                         const float* __restrict__ kernel,
@@ -359,10 +474,31 @@ bool launch_mask_softmax(void* scores, int elt, const int* mask, int B, int rows
     }
     if (!scores) { set_error("softmax: null operand"); return false; }
     const long rows = (long)B * rows_per_batch;
+    unsigned char* sc = static_cast<unsigned char*>(scores);
+    if (elt != kBF16 && elt != kF32) { set_error("softmax: bad element type"); return false; }
+    const int es = elt == kBF16 ? 2 : 4;
+    if ((S * es) % 16 == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0 &&
+        (!mask || (reinterpret_cast<uintptr_t>(mask) & 15) == 0)) {
+        const int chunks = S * es / 16;
+        const int u = chunks > 64 ? 2 : 1;
+        int lpr = 8;
+        while (lpr * u < chunks) lpr *= 2;
+        const int ru = u == 1 ? 4 : 2;
+        const long per_wave = (long)(64 / lpr) * ru;
+        const long waves = (rows + per_wave - 1) / per_wave;
+        const long nblk = (waves + 3) / 4;
+        if (nblk > 0x7fffffffL) { set_error("softmax: too many rows"); return false; }
+        dim3 g((unsigned)nblk), blk(256);
+        if (elt == kBF16 && u == 1) hipLaunchKernelGGL((mask_softmax_vec_kernel<kBF16, 1, 4>), g, blk, 0, stream, sc, mask, rows, rows_per_batch, S, scale, lpr);
+        else if (elt == kBF16) hipLaunchKernelGGL((mask_softmax_vec_kernel<kBF16, 2, 2>), g, blk, 0, stream, sc, mask, rows, rows_per_batch, S, scale, lpr);
+        else if (u == 1) hipLaunchKernelGGL((mask_softmax_vec_kernel<kF32, 1, 4>), g, blk, 0, stream, sc, mask, rows, rows_per_batch, S, scale, lpr);
+        else hipLaunchKernelGGL((mask_softmax_vec_kernel<kF32, 2, 2>), g, blk, 0, stream, sc, mask, rows, rows_per_batch, S, scale, lpr);
+        CUBERT_HIP_OK(hipGetLastError());
+        return true;
+    }
     const long blocks = (rows + 3) / 4;
     if (blocks > 0x7fffffffL) { set_error("softmax: too many rows"); return false; }
     dim3 grid((unsigned)blocks), block(256);
-    unsigned char* sc = static_cast<unsigned char*>(scores);
     if (elt == kBF16) hipLaunchKernelGGL(mask_softmax_kernel<kBF16>, grid, block, 0, stream, sc, mask, rows, rows_per_batch, S, scale);
     else if (elt == kF32) hipLaunchKernelGGL(mask_softmax_kernel<kF32>, grid, block, 0, stream, sc, mask, rows, rows_per_batch, S, scale);
     else { set_error("softmax: bad element type"); return false; }

@@ -276,7 +276,7 @@ def test_embed_layernorm(pb):
 
 
 @pytest.mark.parametrize("elt", [F32, BF16])
-@pytest.mark.parametrize("B,R,S", [(2, 6, 5), (3, 2 * 33, 33), (2, 4 * 200, 200), (1, 512, 512)])
+@pytest.mark.parametrize("B,R,S", [(2, 6, 5), (3, 2 * 33, 33), (2, 4 * 200, 200), (1, 512, 512), (3, 7, 8), (2, 5, 64), (5, 3, 128), (1, 9, 384)])
 def test_mask_softmax(pb, elt, B, R, S):
     rng = np.random.default_rng(S)
     sc = (rng.standard_normal((B, R, S)) * 3).astype(np.float32)
