@@ -153,3 +153,44 @@ def dims_from_npy(npy: Dict[str, np.ndarray], heads: int | None = None) -> BertD
                     vocab=word.shape[0],
                     max_pos=npy["bert_embeddings_position_embeddings"].shape[0],
                     type_vocab=npy["bert_embeddings_token_type_embeddings"].shape[0])
+
+
+def export_checkpoint(init_checkpoint: str, output_dir: str) -> Dict[str, tuple]:
+    """PyTorch checkpoint file -> weight directory; the command-line tool of the reference
+    (convert_pytorch_model_to_npys.py:57-68).  The file is read with
+    ``torch.load(..., weights_only=True)``: only tensors, nothing executed.  Every
+    tensor of the checkpoint is written (task heads included, as the reference does);
+    the engine picks the ones it needs.  Returns {file name: shape}."""
+    import torch
+    sd = torch.load(init_checkpoint, map_location="cpu", weights_only=True)
+    if isinstance(sd, dict) and "state_dict" in sd and isinstance(sd["state_dict"], dict):
+        sd = sd["state_dict"]
+    state = {}
+    for name, t in sd.items():
+        if not torch.is_tensor(t):
+            raise ValueError("checkpoint entry %r is not a tensor" % name)
+        if t.is_floating_point():
+            state[name] = t.detach().to(torch.float32).numpy()
+    export_npy_dir(state, output_dir)
+    return {n: a.shape for n, a in to_npy_layout(state).items()}
+
+
+def main(argv=None) -> int:
+    import argparse
+    ap = argparse.ArgumentParser(description="Write a PyTorch BERT checkpoint as the engine's .npy weight directory")
+    ap.add_argument("--init_checkpoint", default="pytorch_model.bin", help="PyTorch checkpoint (state dict)")
+    ap.add_argument("--output_dir", default="./model_npy", help="directory for the .npy files")
+    ap.add_argument("--check", nargs=4, type=int, metavar=("HIDDEN", "LAYERS", "HEADS", "INTERMEDIATE"),
+                    help="validate the written directory against these model dimensions (needs the built library)")
+    args = ap.parse_args(argv)
+    for name, shape in export_checkpoint(args.init_checkpoint, args.output_dir).items():
+        print(name, " shape : ", tuple(shape))
+    if args.check:
+        from . import pybert
+        pybert.check_weight_dir(args.output_dir, *args.check)
+        print("weight directory accepted for", args.check)
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

@@ -47,3 +47,31 @@ def test_stock_init_statistics():
     assert (sd["bert.embeddings.LayerNorm.weight"] == 1).all()
     w = sd["bert.embeddings.word_embeddings.weight"]
     assert abs(w.std() - 0.02) < 2e-3 and abs(w.mean()) < 2e-3
+
+
+def test_checkpoint_exporter_cli(tmp_path):
+    """A PyTorch checkpoint with the usual `bert.` prefix and pre-training heads goes through the
+    command-line exporter and the library's host-side validation accepts the result."""
+    import torch
+    from cudabert_amd import pybert
+    D = W.TINY
+    state = W.synth_state(D, seed=5)
+    sd = {k: torch.from_numpy(v) for k, v in state.items()}
+    sd["cls.predictions.transform.dense.weight"] = torch.randn(D.hidden, D.hidden)
+    sd["cls.predictions.transform.LayerNorm.weight"] = torch.ones(D.hidden)
+    sd["cls.predictions.transform.LayerNorm.bias"] = torch.zeros(D.hidden)
+    sd["cls.predictions.decoder.weight"] = torch.randn(D.vocab, D.hidden)
+    sd["cls.seq_relationship.weight"] = torch.randn(2, D.hidden)
+    sd["bert.embeddings.position_ids"] = torch.arange(D.max_pos)[None]          # integer buffer: skipped
+    ck = str(tmp_path / "pytorch_model.bin")
+    torch.save(sd, ck)
+    out = str(tmp_path / "npy")
+    assert W.main(["--init_checkpoint", ck, "--output_dir", out, "--check", str(D.hidden), str(D.layers),
+                   str(D.heads), str(D.inter)]) == 0
+    npy = W.load_npy_dir(out)
+    assert npy["cls_predictions_decoder_kernel"].shape == (D.hidden, D.vocab)      # 2-D, not an embedding: transposed
+    assert npy["cls_predictions_transform_LayerNorm_gamma"].shape == (D.hidden,)
+    assert "bert_embeddings_position_ids" not in npy
+    q = "bert.encoder.layer.1.attention.self.query.weight"
+    assert np.array_equal(npy["bert_encoder_layer_1_attention_self_query_kernel"], state[q].T)
+    assert W.dims_from_npy(npy) == D
