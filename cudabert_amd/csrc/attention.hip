@@ -30,7 +30,8 @@ template <int ELT>
 __global__ __launch_bounds__(256) void attention_kernel(
     const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
     const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
-    unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale, int ctx_packed) {
+    unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale, int ctx_packed,
+    const int* __restrict__ cu) {
     constexpr int ES = (ELT == kBF16) ? 2 : 4;
     constexpr int ROWB = 64 * ES;            // bytes per Q/K row
     constexpr int KK = ROWB / 32;            // MFMA k-steps over the head dim (4 bf16 / 8 f32)
@@ -39,7 +40,10 @@ __global__ __launch_bounds__(256) void attention_kernel(
     const int l32 = lane & 31, g = lane >> 5;
     const int h = blockIdx.y, b = blockIdx.z;
     const int q0 = (blockIdx.x * 4 + wave) * 32;
-    if (q0 >= S) return;                      // whole wave leaves; no barriers below
+    // compact rows: only queries below the sequence's length exist, at rows cu[b] + query
+    const int qlen = cu ? cu[b + 1] - cu[b] : S;
+    const size_t row_base = cu ? (size_t)cu[b] : (size_t)b * S;
+    if (q0 >= qlen) return;                   // whole wave leaves; no barriers below
 
     const size_t bh = (size_t)b * heads + h;
     const unsigned char* qb = q + bh * S * ROWB;
@@ -147,10 +151,10 @@ __global__ __launch_bounds__(256) void attention_kernel(
 
     // ---- normalise and store: lane owns query q0 + l32, features 32 db + 8 j + 4 g + e ----
     const int qi = q0 + l32;
-    if (qi >= S) return;
+    if (qi >= qlen) return;
     const float inv = 1.0f / run_sum;
     const size_t hidden = (size_t)heads * 64;
-    unsigned char* orow = ctx + (((size_t)b * S + qi) * hidden + (size_t)h * 64) * ES;
+    unsigned char* orow = ctx + ((row_base + qi) * hidden + (size_t)h * 64) * ES;
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -160,7 +164,7 @@ __global__ __launch_bounds__(256) void attention_kernel(
                 bf16x4_t w = {(__bf16)(o[db][4 * j] * inv), (__bf16)(o[db][4 * j + 1] * inv),
                               (__bf16)(o[db][4 * j + 2] * inv), (__bf16)(o[db][4 * j + 3] * inv)};
                 if (ctx_packed)
-                    *reinterpret_cast<bf16x4_t*>(ctx + packed_offset(b * S + qi, (h * 64 + d) * 2, (int)hidden * 2 / 64)) = w;
+                    *reinterpret_cast<bf16x4_t*>(ctx + packed_offset((int)row_base + qi, (h * 64 + d) * 2, (int)hidden * 2 / 64)) = w;
                 else
                     *reinterpret_cast<bf16x4_t*>(orow + d * 2) = w;
             } else {
@@ -190,7 +194,8 @@ __global__ __launch_bounds__(256) void attention_kernel(
 __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
     const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
-    unsigned char* __restrict__ ctx, int heads, int S, int Sp, int vstride, float scale_log2e, int ctx_packed) {
+    unsigned char* __restrict__ ctx, int heads, int S, int Sp, int vstride, float scale_log2e, int ctx_packed,
+    const int* __restrict__ cu) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* sK = smem;
     unsigned char* sV = smem + (size_t)Sp * 128;
@@ -237,8 +242,12 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 
     // Q fragments ("B" operand: column = query), kept for the whole key loop.
     const int q0 = wave * 32;
+    // compact rows: only queries below the sequence's length exist, at rows cu[b] + query
+    const int qlen = cu ? cu[b + 1] - cu[b] : S;
+    const size_t row_base = cu ? (size_t)cu[b] : (size_t)b * S;
+    if (q0 >= qlen) return;                   // past the last barrier: a whole wave may leave
     int qrow = q0 + l32;
-    qrow = qrow < S ? qrow : S - 1;
+    qrow = qrow < qlen ? qrow : qlen - 1;
     uint4 qf[4];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
@@ -314,10 +323,10 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 
     // ---- normalise and store: lane owns query q0 + l32, features 32 db + 8 j + 4 g + e ----
     const int qi = q0 + l32;
-    if (qi >= S) return;
+    if (qi >= qlen) return;
     const float inv = 1.0f / run_sum;
     const size_t hidden = (size_t)heads * 64;
-    unsigned char* orow = ctx + (((size_t)b * S + qi) * hidden + (size_t)h * 64) * 2;
+    unsigned char* orow = ctx + ((row_base + qi) * hidden + (size_t)h * 64) * 2;
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -326,7 +335,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
             bf16x4_t w = {(__bf16)(o[db][4 * j] * inv), (__bf16)(o[db][4 * j + 1] * inv),
                           (__bf16)(o[db][4 * j + 2] * inv), (__bf16)(o[db][4 * j + 3] * inv)};
             if (ctx_packed)
-                *reinterpret_cast<bf16x4_t*>(ctx + packed_offset(b * S + qi, (h * 64 + d) * 2, (int)hidden * 2 / 64)) = w;
+                *reinterpret_cast<bf16x4_t*>(ctx + packed_offset((int)row_base + qi, (h * 64 + d) * 2, (int)hidden * 2 / 64)) = w;
             else
                 *reinterpret_cast<bf16x4_t*>(orow + d * 2) = w;
         }
@@ -335,7 +344,8 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 }  // namespace
 
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
-                      bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream) {
+                      bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream,
+                      const int* cu) {
     if (ctx_packed && elt != kBF16) { set_error("attention: only a bf16 context can be packed"); return false; }
     const int cp = ctx_packed ? 1 : 0;
     if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
@@ -368,15 +378,15 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
             if (dev >= 0 && dev < 64) allowed[dev] = true;
         }
         hipLaunchKernelGGL(attention_lds_kernel, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd, cc,
-                           heads, S, Sp, vstride, scale * 1.4426950408889634f, cp);
+                           heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);
         CUBERT_HIP_OK(hipGetLastError());
         return true;
     }
     dim3 grid((S + 127) / 128, heads, B), block(256);
     if (elt == kBF16)
-        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp);
+        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu);
     else
-        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp);
+        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }

@@ -54,6 +54,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.graph_max_tokens = cfg.graph_max_tokens;
     opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
     opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
+    opt.varlen = env_int("CUBERT_VARLEN", 0) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;
@@ -142,6 +143,14 @@ int cubert_forward_device(void* model, const int* d_words, const int* d_token_ty
     Model* m = as_model(model, "cubert_forward_device");
     if (!m) return 1;
     return m->forward_device(d_words, d_token_types, d_attention_mask, batchsize, seq_length) ? 0 : 1;
+}
+
+int cubert_forward_device_lens(void* model, const int* d_words, const int* d_token_types, const int* lengths,
+                               int batchsize, int seq_length) {
+    cubert::set_error("");
+    Model* m = as_model(model, "cubert_forward_device_lens");
+    if (!m) return 1;
+    return m->forward_device_lens(d_words, d_token_types, lengths, batchsize, seq_length) ? 0 : 1;
 }
 
 int cubert_classify(void* model) {

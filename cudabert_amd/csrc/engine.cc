@@ -45,6 +45,7 @@ Model::~Model() {
     if (wblock_) (void)hipFree(wblock_);
     if (ablock_) (void)hipFree(ablock_);
     if (h_in_) (void)hipHostFree(h_in_);
+    if (h_meta_) (void)hipHostFree(h_meta_);
     if (ev_fork_) (void)hipEventDestroy(ev_fork_);
     for (int i = 1; i < kMaxParts; ++i) {
         if (ev_join_[i]) (void)hipEventDestroy(ev_join_[i]);
@@ -191,6 +192,8 @@ bool Model::init(const ModelOptions& opt_in) {
     const size_t o_h = aa.take(N * I * es), o_y = aa.take(N * H * 4);
     const size_t o_mask = aa.take(Npad * 4), o_pool = aa.take((size_t)1024 * H * 4), o_cls = aa.take(1024 * 8 * 4);
     const size_t o_in = aa.take(3 * N * 4);
+    const size_t meta_ints = N + (size_t)kMaxParts * kCuStride;
+    const size_t o_meta = aa.take(meta_ints * 4), o_seqpad = aa.take(N * H * 4);
     act_bytes_ = aa.off;
     size_t free_b = 0, total_b = 0;
     CUBERT_HIP_OK(hipMemGetInfo(&free_b, &total_b));
@@ -211,6 +214,9 @@ bool Model::init(const ModelOptions& opt_in) {
     pooled_ = reinterpret_cast<float*>(ablock_ + o_pool);
     cls_ = reinterpret_cast<float*>(ablock_ + o_cls);
     d_in_ = reinterpret_cast<int*>(ablock_ + o_in);
+    d_meta_ = reinterpret_cast<int*>(ablock_ + o_meta);
+    seqpad_ = reinterpret_cast<float*>(ablock_ + o_seqpad);
+    CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_meta_), meta_ints * 4, hipHostMallocDefault));
     CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_in_), 3 * N * 4, hipHostMallocDefault));
     CUBERT_HIP_OK(hipStreamSynchronize(stream_));
     return true;
@@ -258,7 +264,92 @@ bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B,
     CUBERT_HIP_OK(hipMemcpyAsync(d_in_, h_in_, n * 4, hipMemcpyHostToDevice, stream_));
     CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + cap, h_in_ + cap, n * 4, hipMemcpyHostToDevice, stream_));
     if (mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, h_in_ + 2 * cap, n * 4, hipMemcpyHostToDevice, stream_));
+    if (opt_.varlen && mask) {
+        // masks that are 1 on a non-empty prefix and 0 after it: compute the valid tokens only
+        std::vector<int> lens(B);
+        bool prefix = true;
+        for (int b = 0; b < B && prefix; ++b) {
+            const int* m = mask + (size_t)b * S;
+            int len = 0;
+            while (len < S && m[len] == 1) ++len;
+            for (int s = len; s < S && prefix; ++s) prefix = m[s] == 0;
+            prefix = prefix && len >= 1;
+            lens[b] = len;
+        }
+        if (prefix) return run_compact(lens.data(), B, S);
+    }
     return run(B, S, mask != nullptr);
+}
+
+bool Model::forward_device_lens(const int* d_ids, const int* d_seg, const int* h_lens, int B, int S) {
+    if (!check_shape(B, S)) return false;
+    if (!d_ids || !d_seg || !h_lens) { set_error("input_ids, token_type_ids and lengths must not be null"); return false; }
+    for (int b = 0; b < B; ++b)
+        if (h_lens[b] < 1 || h_lens[b] > S) {
+            set_error("length " + std::to_string(h_lens[b]) + " of sequence " + std::to_string(b) + " is outside 1.." + std::to_string(S));
+            return false;
+        }
+    const size_t n = (size_t)B * S, cap = (size_t)cap_tokens_;
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_, d_ids, n * 4, hipMemcpyDeviceToDevice, stream_));
+    CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + cap, d_seg, n * 4, hipMemcpyDeviceToDevice, stream_));
+    return run_compact(h_lens, B, S);
+}
+
+// Unpadded pass: the host lays out, per part, the token index of every compact row and the
+// row offset of every sequence, uploads both and enqueues the parts (never through a graph:
+// the row counts change from call to call).
+bool Model::run_compact(const int* lens, int B, int S) {
+    B_ = B;
+    S_ = S;
+    last_compact_ = true;
+    const long tokens = (long)B * S;
+    int parts = opt_.split_parts < kMaxParts ? opt_.split_parts : kMaxParts;
+    if (parts > B) parts = B;
+    if (parts < 1 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens) parts = 1;
+    // the pinned metadata of the previous call must have been consumed
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    const size_t cap = (size_t)cap_tokens_;
+    // packed operands pad every part to 256 rows; capacity was sized for kMaxParts such regions
+    Compact cp[kMaxParts];
+    size_t r0[kMaxParts];
+    int b0s[kMaxParts], Bs[kMaxParts];
+    size_t rows_total = 0, r = 0;
+    for (int i = 0, b0 = 0; i < parts; ++i) {
+        const int Bi = B / parts + (i < B % parts ? 1 : 0);
+        int* rowmap = h_meta_ + rows_total;
+        int* cu = h_meta_ + cap + 256 * (kMaxParts - 1) + (size_t)i * kCuStride;
+        int rows = 0;
+        for (int b = 0; b < Bi; ++b) {
+            cu[b] = rows;
+            for (int s = 0; s < lens[b0 + b]; ++s) rowmap[rows++] = b * S + s;
+        }
+        cu[Bi] = rows;
+        cp[i].rowmap = d_meta_ + rows_total;
+        cp[i].cu = d_meta_ + cap + 256 * (kMaxParts - 1) + (size_t)i * kCuStride;
+        cp[i].rows = rows;
+        r0[i] = r;
+        b0s[i] = b0;
+        Bs[i] = Bi;
+        rows_total += rows;
+        r += (size_t)round_up(rows, 256);
+        b0 += Bi;
+    }
+    CUBERT_HIP_OK(hipMemcpyAsync(d_meta_, h_meta_, rows_total * 4, hipMemcpyHostToDevice, stream_));
+    const size_t cu_off = cap + 256 * (kMaxParts - 1);
+    CUBERT_HIP_OK(hipMemcpyAsync(d_meta_ + cu_off, h_meta_ + cu_off, (size_t)parts * kCuStride * 4, hipMemcpyHostToDevice, stream_));
+    if (parts == 1) return enqueue_part(0, B, 0, S, false, stream_, &cp[0]);
+    CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
+    bool ok = true;
+    for (int i = 0; i < parts; ++i) {
+        hipStream_t st = i == 0 ? stream_ : side_[i];
+        if (i > 0) CUBERT_HIP_OK(hipStreamWaitEvent(st, ev_fork_, 0));
+        ok = ok && enqueue_part(b0s[i], Bs[i], r0[i], S, false, st, &cp[i]);
+        if (i > 0) {
+            CUBERT_HIP_OK(hipEventRecord(ev_join_[i], st));
+            CUBERT_HIP_OK(hipStreamWaitEvent(stream_, ev_join_[i], 0));
+        }
+    }
+    return ok;
 }
 
 bool Model::forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S) {
@@ -274,6 +365,7 @@ bool Model::forward_device(const int* d_ids, const int* d_seg, const int* d_mask
 bool Model::run(int B, int S, bool has_mask) {
     B_ = B;
     S_ = S;
+    last_compact_ = false;
     const long tokens = (long)B * S;
     if (opt_.graph_max_tokens <= 0 || tokens > opt_.graph_max_tokens) return enqueue(B, S, has_mask);
     const long key = ((long)B * 1024 + S) * 2 + (has_mask ? 1 : 0);
@@ -332,14 +424,16 @@ bool Model::enqueue(int B, int S, bool has_mask) {
 // this part in the internal activation buffers (a multiple of 256, so that a
 // packed operand starts on a block boundary); inputs and the sequence output
 // are indexed by token.
-bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st) {
+bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp) {
     const Dims& D = opt_.dims;
     const int elt = opt_.precision;
     const size_t es = elt == kBF16 ? 2 : 4;
-    const int H = D.hidden, I = D.inter, N = B * S, Sp = round_up(S, 32);
+    // rows of this part: every token, or (unpadded pass) the valid ones only, stored from row r0
+    const int H = D.hidden, I = D.inter, N = cp ? cp->rows : B * S, Sp = round_up(S, 32);
     const size_t cap = (size_t)cap_tokens_, t0 = (size_t)b0 * S;
+    const int* cu = cp ? cp->cu : nullptr;
     const int *ids = d_in_ + t0, *seg = d_in_ + cap + t0, *mask = has_mask ? d_in_ + 2 * cap + t0 : nullptr;
-    float* x32 = x32_ + t0 * H;
+    float* x32 = x32_ + (cp ? r0 : t0) * H;
     float* y32 = y32_ + r0 * H;
     bf16_t* xb = xb_ ? xb_ + r0 * H : nullptr;
     unsigned char* q = static_cast<unsigned char*>(q_) + t0 * H * es;
@@ -354,7 +448,7 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
     if (!mark(kPhEmbed)) return false;
     const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
     if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32, xb, pk, maskadd, B, S, Sp,
-                                H, D.vocab, D.type_vocab, st))
+                                H, D.vocab, D.type_vocab, st, cp))
         return false;
     for (int i = 0; i < D.layers; ++i) {
         const LayerDev& L = layers_[i];
@@ -363,10 +457,11 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         // QKV projection, scattered per head (V transposed)
         g.X = xin; g.ldx = H; g.W = L.w_qkv; g.bias = L.b_qkv; g.M = N; g.N = 3 * H; g.K = H;
         g.epilogue = kEpiQKV; g.q = q; g.k = k; g.vt = vt; g.S = S; g.Sp = Sp; g.heads = D.heads;
+        g.rowmap = cp ? cp->rowmap : nullptr;
         g.x_packed = g.w_packed = pk;
         if (!mark(kPhQKV) || !launch_gemm(g, st)) return false;
         if (!mark(kPhAttention)) return false;
-        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st)) return false;
+        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st, cu)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;
@@ -388,7 +483,9 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
     }
     // pooler: first-token gather + dense + tanh on the float32 sequence output
     if (!mark(kPhPooler)) return false;
-    return launch_pooler(x32, w_pool_, elt, b_pool_, pooled_ + (size_t)b0 * H, B, S, H, st);
+    if (!launch_pooler(x32, w_pool_, elt, b_pool_, pooled_ + (size_t)b0 * H, B, S, H, st, cu)) return false;
+    // unpadded pass: the caller still gets a padded [B, S, H] sequence output
+    return cp ? launch_unpad_rows(x32, cu, seqpad_ + t0 * H, B, S, H, st) : true;
 }
 
 bool Model::mark(int phase) {
@@ -414,6 +511,7 @@ bool Model::profile_device(const int* d_ids, const int* d_seg, const int* d_mask
     if (d_mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, d_mask, n * 4, hipMemcpyDeviceToDevice, stream_));
     B_ = B;
     S_ = S;
+    last_compact_ = false;
     profiling_ = true;
     prof_used_ = 0;
     prof_phase_.clear();
@@ -450,7 +548,7 @@ bool Model::copy_pooled(float* out) {
 
 bool Model::copy_seq(float* out) {
     if (!out || B_ <= 0) { set_error("no result to copy"); return false; }
-    CUBERT_HIP_OK(hipMemcpyAsync(out, x32_, (size_t)B_ * S_ * opt_.dims.hidden * 4, hipMemcpyDeviceToHost, stream_));
+    CUBERT_HIP_OK(hipMemcpyAsync(out, seq_ptr(), (size_t)B_ * S_ * opt_.dims.hidden * 4, hipMemcpyDeviceToHost, stream_));
     return sync();
 }
 

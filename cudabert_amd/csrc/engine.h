@@ -16,6 +16,8 @@
 
 namespace cubert {
 
+struct Compact;      // kernels.h
+
 struct ModelOptions {
     Dims dims;
     int precision = kF32;      // operand type of the GEMMs and attention
@@ -24,6 +26,7 @@ struct ModelOptions {
     int max_seq = 0;
     int split_parts = 2;           // number of parts (1..4) a large batch is cut into
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
+    bool varlen = false;           // host-input calls with prefix masks compute only the valid tokens
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
     std::string dir;
 };
@@ -43,6 +46,11 @@ class Model {
     bool forward_host(const int* ids, const int* seg, const int* mask, int B, int S);
     // Inputs already in device memory.  Asynchronous on stream().
     bool forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S);
+    // Unpadded forward: only the first h_lens[b] >= 1 tokens of every sequence are computed (as if
+    // the attention mask were 1 on exactly those).  Pooled output and the sequence output on
+    // the valid positions equal forward_device's bit for bit; the padding positions of the
+    // sequence output are zero.  h_lens is host memory.  Asynchronous after the metadata upload.
+    bool forward_device_lens(const int* d_ids, const int* d_seg, const int* h_lens, int B, int S);
     // softmax(pooled @ classifier_kernel + bias) for the last forward -> cls_probs().
     bool classify();
     // One eager forward pass with a hipEvent before every launch; fills
@@ -55,7 +63,7 @@ class Model {
     bool copy_seq(float* host_out);                    // D2H + sync, B*S*hidden floats
     bool copy_cls(float* host_out);                    // D2H + sync, B*num_classes floats
 
-    float* seq_ptr() const { return x32_; }
+    float* seq_ptr() const { return last_compact_ ? seqpad_ : x32_; }
     float* pooled_ptr() const { return pooled_; }
     float* cls_ptr() const { return cls_; }
     hipStream_t stream() const { return stream_; }
@@ -75,7 +83,8 @@ class Model {
     bool check_shape(int B, int S);
     bool run(int B, int S, bool has_mask);             // graph or eager
     bool enqueue(int B, int S, bool has_mask);         // the launch sequence (one or two parts)
-    bool enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st);
+    bool enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp = nullptr);
+    bool run_compact(const int* h_lens, int B, int S);
     bool mark(int phase);                              // profiling: event before a launch
 
     ModelOptions opt_;
@@ -105,6 +114,12 @@ class Model {
     float* cls_ = nullptr;       // [B, C]
     int* d_in_ = nullptr;        // ids | seg | mask, cap_tokens each
     int* h_in_ = nullptr;        // pinned staging, same layout
+    // unpadded passes: per part a row map (token index of every compact row) and cu (row offsets)
+    static constexpr int kCuStride = 1032;    // B <= 1024 per part, + 1
+    int* d_meta_ = nullptr;      // rowmap (cap tokens) | cu (kMaxParts * kCuStride)
+    int* h_meta_ = nullptr;      // pinned, same layout
+    float* seqpad_ = nullptr;    // padded [B, S, H] sequence output of an unpadded pass
+    bool last_compact_ = false;
     int B_ = 0, S_ = 0;
     struct GraphEntry { hipGraphExec_t exec = nullptr; int seen = 0; };
     std::map<long, GraphEntry> graphs_;

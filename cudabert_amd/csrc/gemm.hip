@@ -201,6 +201,7 @@ bool launch_epi(const GemmDev& d, int epi, int bt, hipStream_t stream) {
         case kEpiBiasGelu: return launch_tile<ELT, OUT, kEpiBiasGelu>(d, bt, stream);
         case kEpiBiasTanh: return launch_tile<ELT, OUT, kEpiBiasTanh>(d, bt, stream);
         case kEpiQKV: return launch_tile<ELT, OUT, kEpiQKV>(d, bt, stream);
+        case kEpiQKVMap: return launch_tile<ELT, OUT, kEpiQKVMap>(d, bt, stream);
     }
     set_error("gemm: unknown epilogue");
     return false;
@@ -250,9 +251,11 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     d.M = p.M; d.N = p.N; d.K = p.K; d.ldx = p.ldx;
     d.x_packed = p.x_packed; d.w_packed = p.w_packed; d.y_packed = p.y_packed;
     int out = p.out_elt;
+    const int epi = (p.epilogue == kEpiQKV && p.rowmap) ? (int)kEpiQKVMap : p.epilogue;
+    if (p.epilogue == kEpiQKVMap) { set_error("gemm: unknown epilogue"); return false; }
     if (p.epilogue == kEpiQKV) {
         if (!p.q || !p.k || !p.vt || p.S <= 0 || p.heads <= 0 || p.N != 3 * p.heads * 64 ||
-            p.M % p.S != 0 || p.Sp < p.S || p.Sp % 4 != 0) {
+            (!p.rowmap && p.M % p.S != 0) || p.Sp < p.S || p.Sp % 4 != 0) {
             set_error("gemm: bad QKV epilogue arguments");
             return false;
         }
@@ -260,6 +263,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         d.k = static_cast<unsigned char*>(p.k);
         d.vt = static_cast<unsigned char*>(p.vt);
         d.S = p.S; d.Sp = p.Sp; d.heads = p.heads; d.hidden = p.heads * 64;
+        d.rowmap = p.rowmap;
         d.y_packed = 0;
         out = p.elt;
     } else {
@@ -276,12 +280,12 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     if (p.elt == kBF16) {
         // 256 tile with a multiple of four half-steps: the hand-scheduled kernel
         if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled)
-            return launch_gemm_bf16_t256(d, out, p.epilogue, stream);
-        return out == kBF16 ? launch_epi<kBF16, kBF16>(d, p.epilogue, bt, stream)
-                            : launch_epi<kBF16, kF32>(d, p.epilogue, bt, stream);
+            return launch_gemm_bf16_t256(d, out, epi, stream);
+        return out == kBF16 ? launch_epi<kBF16, kBF16>(d, epi, bt, stream)
+                            : launch_epi<kBF16, kF32>(d, epi, bt, stream);
     }
     if (out != kF32) { set_error("gemm: f32 operands require f32 output"); return false; }
-    return launch_epi<kF32, kF32>(d, p.epilogue, bt, stream);
+    return launch_epi<kF32, kF32>(d, epi, bt, stream);
 }
 
 }  // namespace cubert

@@ -99,6 +99,7 @@ bool launch_epi(const GemmDev& d, int epi, hipStream_t stream) {
         case kEpiBiasGelu: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasGelu>), grid, block, 0, stream, d); break;
         case kEpiBiasTanh: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasTanh>), grid, block, 0, stream, d); break;
         case kEpiQKV: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiQKV>), grid, block, 0, stream, d); break;
+        case kEpiQKVMap: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiQKVMap>), grid, block, 0, stream, d); break;
         default: set_error("gemm: unknown epilogue"); return false;
     }
     CUBERT_HIP_OK(hipGetLastError());

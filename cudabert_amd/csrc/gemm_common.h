@@ -24,6 +24,7 @@ struct GemmDev {
     int S, Sp, heads, hidden;
     int tiles_n, tiles_m;
     int x_packed, w_packed, y_packed;     // operand / result in the packed layout (common.h)
+    const int* rowmap;                    // QKV epilogue: row m -> token b * S + s (nullptr: m itself)
 };
 
 __device__ __forceinline__ float gelu_erf(float x) {
@@ -133,14 +134,26 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
     constexpr int EPC = 16 / OES;           // elements per chunk
     const int lane = l32 + 32 * g;
     const int rrow = lane / CH, rc = lane % CH;
+    // compact rows: the token of this lane's row in every block row, fetched together up front;
+    // the read-out phase takes a row's token from the lane that owns it
+    int tokj[NB];
+    if constexpr (EPI == kEpiQKVMap) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int m = m_base + 32 * j + l32;
+            tokj[j] = p.rowmap[m < p.M ? m : p.M - 1];
+        }
+    }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         unsigned char* buf = scratch + ((OES == 2 && (j & 1)) ? 32 * RB : 0);
         const int m = m_base + 32 * j + l32;
         int bidx = 0, sidx = 0;
-        if constexpr (EPI == kEpiQKV) {
-            bidx = m / p.S;
-            sidx = m - bidx * p.S;
+        if constexpr (EPI == kEpiQKV || EPI == kEpiQKVMap) {
+            int tok = m;
+            if constexpr (EPI == kEpiQKVMap) tok = tokj[j];
+            bidx = tok / p.S;
+            sidx = tok - bidx * p.S;
         }
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
@@ -157,7 +170,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                     if constexpr (EPI == kEpiBiasTanh) t = tanhf(t);
                     v[e] = t;
                 }
-                if constexpr (EPI == kEpiQKV) {
+                if constexpr (EPI == kEpiQKV || EPI == kEpiQKVMap) {
                     if (n >= 2 * p.hidden) {
                         if (m < p.M && n < p.N) {
                             const int hn = n - 2 * p.hidden;
@@ -179,10 +192,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             const u32x4_t d = *reinterpret_cast<const u32x4_t*>(buf + row * RB + (((rc ^ row) & (CH - 1)) << 4));
             const int mm = m_base + 32 * j + row;
             const int n = n_base + rc * EPC;
+            int tok = mm;
+            if constexpr (EPI == kEpiQKVMap) tok = __shfl(tokj[j], row);      // before any lane leaves
             if (mm >= p.M || n >= p.N) continue;
-            if constexpr (EPI == kEpiQKV) {
+            if constexpr (EPI == kEpiQKV || EPI == kEpiQKVMap) {
                 if (n >= 2 * p.hidden) continue;
-                const int b2 = mm / p.S, s2 = mm - b2 * p.S;
+                const int b2 = tok / p.S, s2 = tok - b2 * p.S;
                 const int which = n >= p.hidden ? 1 : 0;
                 const int hn = n - which * p.hidden;
                 const size_t bh = (size_t)b2 * p.heads + (hn >> 6);

@@ -22,6 +22,16 @@ enum GemmEpilogue : int {
     kEpiBiasGelu = 1,  // Y = gelu_erf(acc + bias)       (ops/elementwise.cu:37-42 fused)
     kEpiBiasTanh = 2,  // Y = tanh(acc + bias)           (ops/elementwise.cu:56-61 fused)
     kEpiQKV = 3,       // scatter into per-head Q, K and transposed V (see below)
+    kEpiQKVMap = 4,    // the same on compact rows: row m is token rowmap[m] (chosen by launch_gemm when rowmap is set)
+};
+
+// Unpadded ("compact") rows: only the valid tokens of every sequence are stored,
+// sequence after sequence.  rowmap[r] = b * S + s of compact row r; cu[b] = first
+// compact row of sequence b, cu[B] = number of rows.  Both live in device memory.
+struct Compact {
+    const int* rowmap = nullptr;
+    const int* cu = nullptr;
+    int rows = 0;
 };
 
 struct GemmParams {
@@ -41,6 +51,7 @@ struct GemmParams {
     void* k = nullptr;
     void* vt = nullptr;
     int S = 0, Sp = 0, heads = 0;
+    const int* rowmap = nullptr;   // kEpiQKV on compact rows: row m is token rowmap[m] = b * S + s
     int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile)
     bool compiler_scheduled = false;   // 256 tile: use the generic kernel, not the hand-scheduled one
     // Packed operand layout (common.h): X / W read from it, Y (bf16, plain epilogues) written in it.
@@ -59,7 +70,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream);
 // ctx_packed (bf16 only): write ctx in the packed GEMM-operand layout (common.h).
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd,
                       void* ctx, bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt,
-                      hipStream_t stream);
+                      hipStream_t stream, const int* cu = nullptr);
 
 // ----------------------------------------------------------- LayerNorm -----
 // x <- LayerNorm(x + y) * gamma + beta   over rows of length H, in place on the
@@ -80,7 +91,8 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
 bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
                             const float* pos, const float* type, const float* gamma,
                             const float* beta, float* x, bf16_t* xb, bool xb_packed, float* maskadd,
-                            int B, int S, int Sp, int H, int vocab, int type_vocab, hipStream_t stream);
+                            int B, int S, int Sp, int H, int vocab, int type_vocab, hipStream_t stream,
+                            const Compact* compact = nullptr);
 
 // ------------------------------------------------ scale+mask+softmax -------
 // In place over materialised scores [B, rows_per_batch, S] (float32 or bf16):
@@ -101,7 +113,10 @@ bool launch_classifier(const float* pooled, const float* kernel, const float* bi
 // row-major ([out, in]) of type w_elt (cuda_bert/ops/elementwise.cu:5-32, 56-70 and
 // the pooler op_Linear of cuda_bert/utils/bert.cu:238-247; modeling.py:347-353).
 bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, float* pooled, int B, int S, int H,
-                   hipStream_t stream);
+                   hipStream_t stream, const int* cu = nullptr);
+
+// Compact rows -> padded [B, S, H] float32 (zeros on the positions past a sequence's length).
+bool launch_unpad_rows(const float* xc, const int* cu, float* out, int B, int S, int H, hipStream_t stream);
 
 // ------------------------------------------------------ load helpers -------
 // dst[n, k] = convert(src[k, n])  : on-disk [in,out] float32 -> [out,in] operand type,

@@ -105,21 +105,29 @@ __global__ __launch_bounds__(256) void embed_layernorm_kernel(
     const float* __restrict__ word, const float* __restrict__ pos, const float* __restrict__ type,
     const float* __restrict__ gamma, const float* __restrict__ beta, float* __restrict__ x,
     bf16_t* __restrict__ xb, float* __restrict__ maskadd, int B, int S, int Sp, int H, int vocab,
-    int type_vocab, int xb_packed) {
+    int type_vocab, int xb_packed, const int* __restrict__ rowmap, const int* __restrict__ cu, int nrows) {
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= B * S) return;
-    const int b = row / S, s = row - b * S;
-    int id = ids[row];
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);        // output row
+    if (row >= nrows) return;
+    const int tok = rowmap ? rowmap[row] : row;                 // b * S + s
+    const int b = tok / S, s = tok - b * S;
+    int id = ids[tok];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-    int tt = seg ? seg[row] : 0;
+    int tt = seg ? seg[tok] : 0;
     tt = tt < 0 ? 0 : (tt >= type_vocab ? type_vocab - 1 : tt);
     // additive attention mask: 0 valid, -10000 masked, -inf on the padding S..Sp-1
-    if (lane == 0) {
-        const int mk = mask ? mask[row] : 1;
-        maskadd[(size_t)b * Sp + s] = (1.0f - (float)mk) * -10000.0f;
+    if (!rowmap) {
+        if (lane == 0) {
+            const int mk = mask ? mask[tok] : 1;
+            maskadd[(size_t)b * Sp + s] = (1.0f - (float)mk) * -10000.0f;
+        }
+        if (s == 0 && S + lane < Sp) maskadd[(size_t)b * Sp + S + lane] = -INFINITY;   // Sp - S < 32
+    } else if (s == 0) {
+        // compact rows: the first token of a sequence writes the whole mask row from the length
+        const int len = cu[b + 1] - cu[b];
+        for (int i = lane; i < Sp; i += 64)
+            maskadd[(size_t)b * Sp + i] = i < len ? 0.0f : (i < S ? -10000.0f : -INFINITY);
     }
-    if (s == 0 && S + lane < Sp) maskadd[(size_t)b * Sp + S + lane] = -INFINITY;   // Sp - S < 32
     const float* wr = word + (size_t)id * H;
     const float* pr = pos + (size_t)s * H;
     const float* tr = type + (size_t)tt * H;
@@ -374,10 +382,10 @@ __global__ void fill_f32_kernel(float* dst, float value, size_t n) {
 template <int ELT>
 __global__ __launch_bounds__(256) void pooler_kernel(const float* __restrict__ x, const unsigned char* __restrict__ W,
                                                      const float* __restrict__ bias, float* __restrict__ pooled,
-                                                     int S, int H) {
+                                                     int S, int H, const int* __restrict__ cu) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int b = blockIdx.x;
-    const float* xr = x + (size_t)b * S * H;
+    const float* xr = x + (cu ? (size_t)cu[b] : (size_t)b * S) * H;      // first token of sequence b
     float xv[kMaxChunks][4];
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
@@ -412,6 +420,23 @@ __global__ __launch_bounds__(256) void pooler_kernel(const float* __restrict__ x
     }
 }
 
+// out[b, s, :] = s < len(b) ? xc[cu[b] + s, :] : 0; one wave per padded token row.
+__global__ __launch_bounds__(256) void unpad_rows_kernel(const float* __restrict__ xc, const int* __restrict__ cu,
+                                                         float* __restrict__ out, int B, int S, int H) {
+    const int lane = threadIdx.x & 63;
+    const long tok = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tok >= (long)B * S) return;
+    const int b = (int)(tok / S), s = (int)(tok - (long)b * S);
+    const int first = cu[b], len = cu[b + 1] - first;
+    const float* src = xc + (size_t)(first + s) * H;
+    float* dst = out + (size_t)tok * H;
+    for (int i = lane * 4; i < H; i += 256) {
+        f32x4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (s < len) v = *reinterpret_cast<const f32x4_t*>(src + i);
+        *reinterpret_cast<f32x4_t*>(dst + i) = v;
+    }
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
@@ -442,7 +467,11 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
 bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word,
                             const float* pos, const float* type, const float* gamma, const float* beta,
                             float* x, bf16_t* xb, bool xb_packed, float* maskadd, int B, int S, int Sp, int H,
-                            int vocab, int type_vocab, hipStream_t stream) {
+                            int vocab, int type_vocab, hipStream_t stream, const Compact* compact) {
+    if (compact && (!compact->rowmap || !compact->cu || compact->rows <= 0 || compact->rows > (long)B * S)) {
+        set_error("embedding: bad compact-row description");
+        return false;
+    }
     if (xb && xb_packed && H % 32 != 0) { set_error("embedding: a packed copy needs H to be a multiple of 32"); return false; }
     if (B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
         set_error("embedding: H must be a multiple of 4 and at most 1024");
@@ -458,10 +487,11 @@ bool launch_embed_layernorm(const int* ids, const int* seg, const int* mask, con
         set_error("embedding: misaligned operand");
         return false;
     }
-    const long rows = (long)B * S;
+    const long rows = compact ? compact->rows : (long)B * S;
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
     hipLaunchKernelGGL(embed_layernorm_kernel, grid, block, 0, stream, ids, seg, mask, word, pos, type, gamma,
-                       beta, x, xb, maskadd, B, S, Sp, H, vocab, type_vocab, xb_packed ? 1 : 0);
+                       beta, x, xb, maskadd, B, S, Sp, H, vocab, type_vocab, xb_packed ? 1 : 0,
+                       compact ? compact->rowmap : nullptr, compact ? compact->cu : nullptr, (int)rows);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }
@@ -516,7 +546,7 @@ bool launch_classifier(const float* pooled, const float* kernel, const float* bi
 }
 
 bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, float* pooled, int B, int S, int H,
-                   hipStream_t stream) {
+                   hipStream_t stream, const int* cu) {
     if (B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || H > kMaxChunks * 256) {
         set_error("pooler: H must be a multiple of 4 and at most 1024");
         return false;
@@ -525,9 +555,20 @@ bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, 
     if (B > 65535) { set_error("pooler: batch too large"); return false; }
     dim3 grid(B, (H + 63) / 64), block(256);
     const unsigned char* wc = static_cast<const unsigned char*>(W);
-    if (w_elt == kBF16) hipLaunchKernelGGL(pooler_kernel<kBF16>, grid, block, 0, stream, x, wc, bias, pooled, S, H);
-    else if (w_elt == kF32) hipLaunchKernelGGL(pooler_kernel<kF32>, grid, block, 0, stream, x, wc, bias, pooled, S, H);
+    if (w_elt == kBF16) hipLaunchKernelGGL(pooler_kernel<kBF16>, grid, block, 0, stream, x, wc, bias, pooled, S, H, cu);
+    else if (w_elt == kF32) hipLaunchKernelGGL(pooler_kernel<kF32>, grid, block, 0, stream, x, wc, bias, pooled, S, H, cu);
     else { set_error("pooler: bad weight type"); return false; }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_unpad_rows(const float* xc, const int* cu, float* out, int B, int S, int H, hipStream_t stream) {
+    if (!xc || !cu || !out || B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || !aligned16(xc) || !aligned16(out)) {
+        set_error("unpad: bad arguments");
+        return false;
+    }
+    const long rows = (long)B * S;
+    hipLaunchKernelGGL(unpad_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, xc, cu, out, B, S, H);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }

@@ -63,6 +63,8 @@ lib.init_model_ex.argtypes = [POINTER(Config), c_int, c_int, c_int, c_char_p]
 lib.init_model_ex.restype = c_void_p
 lib.cubert_check_weight_dir.argtypes = [POINTER(Config), c_char_p]
 lib.cubert_check_weight_dir.restype = c_int
+lib.cubert_forward_device_lens.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int]
+lib.cubert_forward_device_lens.restype = c_int
 lib.cubert_encode.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]
 lib.cubert_encode.restype = c_int
 lib.cubert_forward_device.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int]

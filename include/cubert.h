@@ -104,6 +104,19 @@ int cubert_forward_device(void* model, const int* d_words, const int* d_token_ty
                           const int* d_attention_mask, int batchsize, int seq_length);
 int cubert_sync(void* model);
 
+/* Unpadded forward pass (goes beyond the reference, which pads every batch to its
+ * longest line, utils.py:3-13): only the first lengths[b] (1..seq_length) tokens of
+ * every sequence are computed, as if the attention mask were 1 on exactly those.
+ * d_words / d_token_types are device [B, S] as above; `lengths` is HOST memory [B].
+ * The pooled output and the sequence output on the valid positions are bit-identical
+ * to cubert_forward_device with the corresponding prefix mask; the sequence output is
+ * zero on the padding positions (the padded pass computes values there that no caller
+ * uses).  The host-input entry points (Cuda_Bert, Cuda_Inference, cubert_encode) take
+ * this path by themselves when CUBERT_VARLEN=1 and every mask row is a non-empty
+ * prefix of ones.  Returns 0 on success. */
+int cubert_forward_device_lens(void* model, const int* d_words, const int* d_token_types,
+                               const int* lengths, int batchsize, int seq_length);
+
 /* Enqueues the fine-tune head on the pooled output of the last forward pass
  * (softmax(pooled @ classifier_kernel + bias), apps/finetune.py:16-44; the
  * reference's commented-out classify_inference, cuda_bert/utils/bert.cu:254-265).

@@ -254,3 +254,55 @@ def test_split_batch_two_streams_is_bit_identical(pb, tiny_dir, precision, monke
     finally:
         for m in (whole, split, split_graph):
             pb.unload_model(m)
+
+
+@pytest.mark.parametrize("precision", [F32, BF16])
+@pytest.mark.parametrize("split", ["0", "1"])
+def test_unpadded_pass_matches_padded_on_valid_positions(pb, tiny_dir, precision, split, monkeypatch):
+    """Computing only the valid tokens (compact rows) gives, bit for bit, the padded pass's pooled
+    output and sequence output on the valid positions, zeros on the padding; through the
+    device entry point with host lengths and through the host entry point with CUBERT_VARLEN=1."""
+    import ctypes
+    wdir = str(tiny_dir / ("f32" if precision == F32 else "bf16"))
+    B, S = 7, 45
+    lens = np.array([45, 1, 20, 33, 2, 45, 17], np.int32)
+    ids, seg, mask = synth.make_inputs(B, S, list(lens), vocab=W.TINY.vocab, seed=5, prune=False)
+    monkeypatch.setenv("CUBERT_SPLIT_MIN_TOKENS", split)
+    padded = load(pb, W.TINY, wdir, precision, B, S)
+    monkeypatch.setenv("CUBERT_VARLEN", "1")
+    compact = load(pb, W.TINY, wdir, precision, B, S)
+    try:
+        pooled0, seq0, cls0 = pb.encode(padded, ids, seg, mask, want_seq=True, want_cls=True)
+        valid = mask.astype(bool)
+        for rep in range(2):
+            pooled1, seq1, cls1 = pb.encode(compact, ids, seg, mask, want_seq=True, want_cls=True)
+            assert np.array_equal(pooled0, pooled1)
+            assert np.array_equal(cls0, cls1)
+            assert np.array_equal(seq0[valid], seq1[valid])
+            assert (seq1[~valid] == 0).all()
+        # a mask with a hole is not a prefix mask: the host path must fall back to the padded pass
+        holed = mask.copy()
+        holed[0, 3] = 0
+        p_ref, s_ref, _ = pb.encode(padded, ids, seg, holed, want_seq=True)
+        p_got, s_got, _ = pb.encode(compact, ids, seg, holed, want_seq=True)
+        assert np.array_equal(p_ref, p_got) and np.array_equal(s_ref, s_got)
+        # device inputs + host lengths
+        d = [torch.from_numpy(a).cuda() for a in (ids, seg)]
+        torch.cuda.synchronize()
+        pb.check(pb.lib.cubert_forward_device_lens(padded, d[0].data_ptr(), d[1].data_ptr(), lens.ctypes.data, B, S))
+        pb.check(pb.lib.cubert_sync(padded))
+        H = W.TINY.hidden
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        pooled2 = np.empty((B, H), np.float32)
+        seq2 = np.empty((B, S, H), np.float32)
+        assert hip.hipMemcpy(pooled2.ctypes.data, pb.lib.cubert_pooled_ptr(padded), pooled2.nbytes, 2) == 0
+        assert hip.hipMemcpy(seq2.ctypes.data, pb.lib.cubert_seq_ptr(padded), seq2.nbytes, 2) == 0
+        assert np.array_equal(pooled0, pooled2)
+        assert np.array_equal(seq0[valid], seq2[valid]) and (seq2[~valid] == 0).all()
+        # bad lengths are refused
+        bad = lens.copy(); bad[2] = 0
+        assert pb.lib.cubert_forward_device_lens(padded, d[0].data_ptr(), d[1].data_ptr(), bad.ctypes.data, B, S) != 0
+    finally:
+        pb.unload_model(padded)
+        pb.unload_model(compact)
