@@ -55,6 +55,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
     opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
     opt.varlen = env_int("CUBERT_VARLEN", 0) != 0;
+    opt.split_k = env_int("CUBERT_SPLIT_K", 1) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;
@@ -252,6 +253,7 @@ void apply_gemm_flags(cubert::GemmParams* p, int flags) {
     p->w_packed = (flags & CUBERT_W_PACKED) != 0;
     p->y_packed = (flags & CUBERT_Y_PACKED) != 0;
     p->compiler_scheduled = (flags & CUBERT_COMPILER_SCHEDULED) != 0;
+    p->splits = CUBERT_SPLITS_OF(flags) > 1 ? CUBERT_SPLITS_OF(flags) : 1;
 }
 }  // namespace
 
@@ -294,7 +296,8 @@ int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gam
     cubert::set_error("");
     return cubert::launch_add_layernorm(x, y, y_elt, gamma, beta, static_cast<cubert::bf16_t*>(xb),
                                         (flags & CUBERT_Y_PACKED) != 0, rows, hidden,
-                                        static_cast<hipStream_t>(stream)) ? 0 : 1;
+                                        static_cast<hipStream_t>(stream),
+                                        CUBERT_SPLITS_OF(flags) > 1 ? CUBERT_SPLITS_OF(flags) : 1) ? 0 : 1;
 }
 
 int cubert_op_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word, const float* pos,

@@ -189,7 +189,7 @@ bool Model::init(const ModelOptions& opt_in) {
     const size_t o_xb = elt == kBF16 ? aa.take(N * H * 2) : 0;
     const size_t o_q = aa.take((N + 64) * H * es), o_k = aa.take((N + 64) * H * es);
     const size_t o_vt = aa.take(Npad * H * es), o_ctx = aa.take(N * H * es);
-    const size_t o_h = aa.take(N * I * es), o_y = aa.take(N * H * 4);
+    const size_t o_h = aa.take(N * I * es), o_y = aa.take((N + kSplitRows) * H * 4);
     const size_t o_mask = aa.take(Npad * 4), o_pool = aa.take((size_t)1024 * H * 4), o_cls = aa.take(1024 * 8 * 4);
     const size_t o_in = aa.take(3 * N * 4);
     const size_t meta_ints = N + (size_t)kMaxParts * kCuStride;
@@ -337,6 +337,7 @@ bool Model::run_compact(const int* lens, int B, int S) {
     CUBERT_HIP_OK(hipMemcpyAsync(d_meta_, h_meta_, rows_total * 4, hipMemcpyHostToDevice, stream_));
     const size_t cu_off = cap + 256 * (kMaxParts - 1);
     CUBERT_HIP_OK(hipMemcpyAsync(d_meta_ + cu_off, h_meta_ + cu_off, (size_t)parts * kCuStride * 4, hipMemcpyHostToDevice, stream_));
+    cur_parts_ = parts;
     if (parts == 1) return enqueue_part(0, B, 0, S, false, stream_, &cp[0]);
     CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
     bool ok = true;
@@ -398,8 +399,11 @@ bool Model::enqueue(int B, int S, bool has_mask) {
     const long tokens = (long)B * S;
     int parts = opt_.split_parts < kMaxParts ? opt_.split_parts : kMaxParts;
     if (parts > B) parts = B;
-    if (profiling_ || parts < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens)
+    if (profiling_ || parts < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens) {
+        cur_parts_ = 1;
         return enqueue_part(0, B, 0, S, has_mask, stream_);
+    }
+    cur_parts_ = parts;
     CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
     bool ok = true;
     size_t r0 = 0;
@@ -445,6 +449,17 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
     const void* xin = elt == kBF16 ? static_cast<const void*>(xb) : static_cast<const void*>(x32);
     const float scale = 1.0f / std::sqrt(64.0f);
 
+    // Short batches: the two GEMMs with only `hidden` output features have too few tiles for the
+    // chip; they split K over several workgroups and the LayerNorm that follows adds the parts.
+    auto splits_for = [&](int K) {
+        const long tiles = (long)((N + 63) / 64) * ((H + 63) / 64);
+        int sp = 1;
+        if (cur_parts_ != 1 || !opt_.split_k) return sp;    // the parts of a split batch sit side by side in y32
+        while (sp < 16 && tiles * sp < 512 && K / (sp * 2) >= 256 && (long)(sp * 2) * N <= (long)N + kSplitRows) sp *= 2;
+        return sp;
+    };
+    const int sp_ao = splits_for(H), sp_fo = splits_for(I);
+
     if (!mark(kPhEmbed)) return false;
     const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
     if (!launch_embed_layernorm(ids, seg, mask, word_, pos_, type_, emb_g_, emb_b_, x32, xb, pk, maskadd, B, S, Sp,
@@ -465,10 +480,10 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;
-        g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
+        g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_ao;
         if (!mark(kPhAttnOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st)) return false;
+        if (!launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st, sp_ao)) return false;
         // feed-forward
         g = GemmParams();
         g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h;
@@ -476,10 +491,10 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         if (!mark(kPhFFNIn) || !launch_gemm(g, st)) return false;
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = h; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32;
-        g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
+        g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_fo;
         if (!mark(kPhFFNOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st)) return false;
+        if (!launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st, sp_fo)) return false;
     }
     // pooler: first-token gather + dense + tanh on the float32 sequence output
     if (!mark(kPhPooler)) return false;

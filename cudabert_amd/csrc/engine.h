@@ -26,6 +26,7 @@ struct ModelOptions {
     int max_seq = 0;
     int split_parts = 2;           // number of parts (1..4) a large batch is cut into
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
+    bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
     bool varlen = false;           // host-input calls with prefix masks compute only the valid tokens
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
     std::string dir;
@@ -115,11 +116,13 @@ class Model {
     int* d_in_ = nullptr;        // ids | seg | mask, cap_tokens each
     int* h_in_ = nullptr;        // pinned staging, same layout
     // unpadded passes: per part a row map (token index of every compact row) and cu (row offsets)
+    static constexpr int kSplitRows = 8192;   // extra rows of y32 for the partial results of split-K GEMMs
     static constexpr int kCuStride = 1032;    // B <= 1024 per part, + 1
     int* d_meta_ = nullptr;      // rowmap (cap tokens) | cu (kMaxParts * kCuStride)
     int* h_meta_ = nullptr;      // pinned, same layout
     float* seqpad_ = nullptr;    // padded [B, S, H] sequence output of an unpadded pass
     bool last_compact_ = false;
+    int cur_parts_ = 1;          // parts of the pass being enqueued
     int B_ = 0, S_ = 0;
     struct GraphEntry { hipGraphExec_t exec = nullptr; int seen = 0; };
     std::map<long, GraphEntry> graphs_;

@@ -95,7 +95,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     const int w_ks = p.w_packed ? 32768 : 128, x_ks = p.x_packed ? 32768 : 128;         // K step strides
 
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
-    const int KT = p.K / BK;
+    // K steps of this workgroup: all of them, or (split K) the blockIdx.y-th share
+    const int steps = p.K / BK;
+    const int kt0 = (int)((long)steps * blockIdx.y / p.splits);
+    const int KT = (int)((long)steps * (blockIdx.y + 1) / p.splits);
     // A K step past the end (odd step counts run one phantom step) fetches from
     // beyond the descriptor's range and therefore fills the tile with zeros.
 #define CUBERT_ISSUE_TILE(BUF, kt)                                                                          \
@@ -159,10 +162,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
         __builtin_amdgcn_sched_barrier(0);                                                                  \
     } while (0)
 
-    CUBERT_ISSUE_TILE(lds0, 0);
+    CUBERT_ISSUE_TILE(lds0, kt0);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    for (int kt = 0; kt < KT; kt += 2) {
+    for (int kt = kt0; kt < KT; kt += 2) {
         CUBERT_K_STEP(lds0, lds1, kt);
         CUBERT_K_STEP(lds1, lds0, kt + 1);
     }
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 
 template <int ELT, int OUT, int EPI, int BT>
 bool launch_one(const GemmDev& d, hipStream_t stream) {
-    hipLaunchKernelGGL((gemm_kernel<ELT, OUT, EPI, BT>), dim3(d.tiles_n * d.tiles_m), dim3(256), 0, stream, d);
+    hipLaunchKernelGGL((gemm_kernel<ELT, OUT, EPI, BT>), dim3(d.tiles_n * d.tiles_m, d.splits), dim3(256), 0, stream, d);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }
@@ -217,7 +220,7 @@ int gemm_pick_tile(int M, int N, int K, int elt) {
     // when its tiles cover well under half of the CUs.
     auto tiles = [&](int bt) { return (long)((M + bt - 1) / bt) * ((N + bt - 1) / bt); };
     if (tiles(256) >= 256) return 256;
-    if (elt == kBF16 && K % 128 == 0 && tiles(256) >= 96) return 256;
+    if (elt == kBF16 && K % 128 == 0 && tiles(256) >= 160) return 256;
     if (tiles(128) >= 256) return 128;
     return 64;
 }
@@ -274,12 +277,20 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
             return false;
         }
     }
-    const int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
+    d.splits = p.splits > 0 ? p.splits : 1;
+    if (d.splits > 1) {
+        if (epi != kEpiBias || out != kF32 || p.y_packed || d.splits > p.K / bk) {
+            set_error("gemm: split K needs the plain bias epilogue, a float32 result and at least one K step per split");
+            return false;
+        }
+    }
+    int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
+    if (d.splits > 1 && bt == 256 && !p.tile) bt = 128;      // the hand-scheduled kernel does not split
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
     if (p.elt == kBF16) {
         // 256 tile with a multiple of four half-steps: the hand-scheduled kernel
-        if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled)
+        if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled && d.splits == 1)
             return launch_gemm_bf16_t256(d, out, epi, stream);
         return out == kBF16 ? launch_epi<kBF16, kBF16>(d, epi, bt, stream)
                             : launch_epi<kBF16, kF32>(d, epi, bt, stream);

@@ -25,6 +25,7 @@ struct GemmDev {
     int tiles_n, tiles_m;
     int x_packed, w_packed, y_packed;     // operand / result in the packed layout (common.h)
     const int* rowmap;                    // QKV epilogue: row m -> token b * S + s (nullptr: m itself)
+    int splits;                           // split K: blockIdx.y owns a K range, results go to Y + y * M * N (f32)
 };
 
 __device__ __forceinline__ float gelu_erf(float x) {
@@ -121,6 +122,7 @@ __device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int
     for (int t = 0; t < 4 * NB; ++t) {
         const int n = n_base + 8 * t + 4 * g;
         bias[t] = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
+        if (blockIdx.y != 0) bias[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};     // split K: the bias is added once
     }
 }
 
@@ -206,7 +208,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 // packed bf16 result: the next GEMM's activation operand
                 *reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)) = d;
             } else {
-                *reinterpret_cast<u32x4_t*>(p.Y + ((size_t)mm * p.N + n) * OES) = d;
+                *reinterpret_cast<u32x4_t*>(p.Y + (((size_t)blockIdx.y * p.M + mm) * p.N + n) * OES) = d;
             }
         }
     }

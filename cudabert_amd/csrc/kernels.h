@@ -53,6 +53,10 @@ struct GemmParams {
     int S = 0, Sp = 0, heads = 0;
     const int* rowmap = nullptr;   // kEpiQKV on compact rows: row m is token rowmap[m] = b * S + s
     int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile)
+    // Split K (kEpiBias, float32 Y): `splits` workgroups share a tile, each reduces its share of K and
+    // writes its partial result to Y + z * M * N; the bias goes into partial 0.  The consumer adds
+    // them up (launch_add_layernorm's y_parts).  Y must hold splits * M * N floats.
+    int splits = 1;
     bool compiler_scheduled = false;   // 256 tile: use the generic kernel, not the hand-scheduled one
     // Packed operand layout (common.h): X / W read from it, Y (bf16, plain epilogues) written in it.
     bool x_packed = false, w_packed = false, y_packed = false;
@@ -81,7 +85,7 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
 // xb_packed: write the copy in the packed GEMM-operand layout (common.h).
 bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
                           const float* beta, bf16_t* xb, bool xb_packed, int rows, int H,
-                          hipStream_t stream);
+                          hipStream_t stream, int y_parts = 1);
 
 // --------------------------------------------------- embedding + LN --------
 // x[t] = LayerNorm(word[ids[t]] + pos[t % S] + type[seg[t]]); also writes the

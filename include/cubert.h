@@ -153,6 +153,11 @@ long cubert_capacity_tokens(void* model);
 #define CUBERT_W_PACKED 2           /* weight operand W is packed */
 #define CUBERT_Y_PACKED 4           /* write Y packed (bf16 output only) */
 #define CUBERT_COMPILER_SCHEDULED 8 /* 256 tile: general kernel instead of the hand-scheduled one */
+/* Split K (cubert_op_gemm, epilogue 0, float32 Y): n workgroups share a tile, each reduces 1/n of K
+ * and writes its partial sum to Y + i * M * N (the bias is in partial 0); Y holds n * M * N floats and
+ * the consumer adds the parts (cubert_op_add_layernorm takes the count in the same flag bits). */
+#define CUBERT_SPLITS(n) (((n) & 0xff) << 8)
+#define CUBERT_SPLITS_OF(flags) (((flags) >> 8) & 0xff)
 size_t cubert_packed_bytes(size_t rows, size_t row_bytes);
 size_t cubert_packed_offset(int row, int byte_in_row, int row_bytes);
 

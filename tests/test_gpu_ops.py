@@ -334,6 +334,46 @@ def test_gemm_packed_operands(pb, tile, flags_extra, M, N, K, epi, xp, wp, yp):
     assert np.abs(got - ref).max() < tol, np.abs(got - ref).max()
 
 
+@pytest.mark.parametrize("elt", [F32, BF16])
+@pytest.mark.parametrize("M,N,K,splits,tile", [(200, 1024, 4096, 4, 64), (77, 128, 512, 2, 0), (300, 256, 1024, 8, 128),
+                                               (64, 64, 384, 3, 64)])
+def test_gemm_split_k_and_layernorm_of_parts(pb, elt, M, N, K, splits, tile):
+    """Split-K GEMM: the partial results add up to the plain product, and the residual+LayerNorm
+    kernel consumes them as its addend."""
+    rng = np.random.default_rng(M + K)
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    Wt = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    tdt = torch.float32 if elt == F32 else torch.bfloat16
+    if elt == BF16:
+        X, Wt = bf16_round(X), bf16_round(Wt)
+    ref = X.astype(np.float64) @ Wt.astype(np.float64).T + b
+    Xd, Wd, bd = dev(X, tdt), dev(Wt, tdt), dev(b)
+    Y = torch.full((splits, M, N), float("nan"), device="cuda")
+    flags = (splits & 0xff) << 8
+    pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), M, N, K, K, elt, F32, 0,
+                                   tile, flags, stream()))
+    torch.cuda.synchronize()
+    parts = Y.cpu().numpy().astype(np.float64)
+    assert np.isfinite(parts).all()
+    assert np.abs(parts.sum(0) - ref).max() < 3e-4 * max(1.0, np.sqrt(K / 512))
+    assert np.abs(parts[1:]).max() > 0                      # the work really was divided
+    # residual + LayerNorm over the parts == over their sum
+    x = rng.standard_normal((M, N)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    be = (0.1 * rng.standard_normal(N)).astype(np.float32)
+    z = x.astype(np.float64) + parts.sum(0)
+    zr = (z - z.mean(-1, keepdims=True)) / np.sqrt(z.var(-1, keepdims=True) + 1e-12) * g + be
+    xd, gd, bed = dev(x), dev(g), dev(be)
+    pb.check(pb.lib.cubert_op_add_layernorm(xd.data_ptr(), Y.data_ptr(), F32, gd.data_ptr(), bed.data_ptr(), None, M, N,
+                                            flags, stream()))
+    torch.cuda.synchronize()
+    assert np.abs(xd.cpu().numpy() - zr).max() < 2e-4
+    # not allowed: GELU epilogue or bf16 result with split K
+    assert pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y.data_ptr(), M, N, K, K, elt, F32, 1,
+                                 tile, flags, stream()) != 0
+
+
 def test_packed_producers(pb):
     """LayerNorm, embedding and attention writing their bf16 result packed."""
     rng = np.random.default_rng(3)
