@@ -24,6 +24,7 @@ def pb():
 def declared_symbols():
     text = open(os.path.join(ROOT, "include", "cubert.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^[ \t]*#.*$", "", text, flags=re.M)          # macros are not symbols
     return sorted(set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\([^;{]*\)\s*;", text)))
 
 
