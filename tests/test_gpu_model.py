@@ -308,3 +308,46 @@ def test_unpadded_pass_matches_padded_on_valid_positions(pb, tiny_dir, precision
     finally:
         pb.unload_model(padded)
         pb.unload_model(compact)
+
+
+def test_large_headline_shape(pb, tmp_path):
+    """BERT-large at the headline shape (batch 128, seq 200, ragged lengths, bf16): the first
+    sequences against the oracle within the bf16 tolerance, and the properties that do not
+    depend on size -- the unpadded pass equals the padded one on valid positions bit for
+    bit, and permuting the batch permutes the outputs."""
+    import ctypes
+    D = W.LARGE
+    state = bf16_exact(W.synth_state(D, seed=20240, degenerate=False))
+    wdir = W.export_npy_dir(state, str(tmp_path / "large"))
+    npy = W.to_npy_layout(state)
+    del state
+    ids, seg, mask = synth.config_inputs(2)
+    B, S = ids.shape
+    lens = np.ascontiguousarray(mask.sum(1).astype(np.int32))
+    m = load(pb, D, wdir, BF16, B, S)
+    try:
+        pooled, seq, cls = pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)
+        n = 3
+        seq_ref, pooled_ref = O.forward_torch(npy, D.heads, ids[:n], seg[:n], mask[:n])
+        assert np.abs(seq[:n] - seq_ref).max() < TOL[BF16]
+        assert np.abs(pooled[:n] - pooled_ref).max() < TOL[BF16]
+        assert np.abs(cls[:n] - O.classifier_head(npy, pooled_ref)).max() < TOL[BF16]
+        assert np.isfinite(seq).all() and np.allclose(cls.sum(1), 1.0, atol=1e-5)
+        perm = np.random.default_rng(1).permutation(B)
+        pooled_p, seq_p, _ = pb.encode(m, ids[perm], seg[perm], mask[perm], want_seq=True)
+        assert np.array_equal(pooled_p, pooled[perm]) and np.array_equal(seq_p, seq[perm])
+        d = [torch.from_numpy(a).cuda() for a in (ids, seg)]
+        torch.cuda.synchronize()
+        pb.check(pb.lib.cubert_forward_device_lens(m, d[0].data_ptr(), d[1].data_ptr(), lens.ctypes.data, B, S))
+        pb.check(pb.lib.cubert_sync(m))
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        pooled_u = np.empty_like(pooled)
+        seq_u = np.empty_like(seq)
+        assert hip.hipMemcpy(pooled_u.ctypes.data, pb.lib.cubert_pooled_ptr(m), pooled_u.nbytes, 2) == 0
+        assert hip.hipMemcpy(seq_u.ctypes.data, pb.lib.cubert_seq_ptr(m), seq_u.nbytes, 2) == 0
+        valid = mask.astype(bool)
+        assert np.array_equal(pooled_u, pooled)
+        assert np.array_equal(seq_u[valid], seq[valid]) and (seq_u[~valid] == 0).all()
+    finally:
+        pb.unload_model(m)
