@@ -4,8 +4,10 @@
 // computes a BT x BT macro tile (BT features x BT tokens), each wave a
 // (BT/2) x (BT/2) quadrant built from 32x32 MFMA blocks.  Per K step a slab of
 // 128 bytes per row (64 bf16 / 32 f32) of both operands is loaded straight
-// from global memory into LDS (buffer_load ... lds, double buffered, one
-// barrier per step).
+// from global memory into LDS (buffer_load ... lds, one barrier per step): two
+// LDS stages for the 256 and 128 tiles, four for the 64 tile, whose steps are so
+// short that a single step of prefetch leaves every step waiting a full memory
+// latency.
 //
 // LDS image of an operand tile: two sub-blocks (the two 64-byte halves of the
 // K slab), each BT rows x 64 bytes; a row is four 16-byte chunks and chunk c
@@ -50,11 +52,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     constexpr int SBDIV = BT / 16;                   // 16-row groups per sub-block
     constexpr int BK = 128 / ES;                     // K elements per step
 
-    // Two separate LDS objects (not one array indexed by parity): the compiler
+    // LDS stages: four for the 64 tile (64 KiB, two workgroups still fit a CU); the 128 tile keeps
+    // two (four would cost it the second resident workgroup), the 256 tile fills the LDS with two.
+    constexpr int NS = (BT == 64) ? 4 : 2;
+    constexpr int LPT = 2 * GROUPS;                  // loads a wave issues per step
+    // s_waitcnt vmcnt(n) with n = the loads of the NS - 2 youngest tiles: the next tile has landed
+    constexpr int WAIT_N = LPT * (NS - 2);
+    constexpr int WAIT_IMM = 0x0F70 | (WAIT_N & 15) | ((WAIT_N >> 4) << 14);
+
+    // Separate LDS objects (not one array indexed by stage): the compiler
     // then knows that the asynchronous global->LDS loads filling one buffer
-    // cannot alias the fragment reads of the other and does not serialise them.
+    // cannot alias the fragment reads of another and does not serialise them.
     __shared__ __attribute__((aligned(1024))) unsigned char lds0[2 * TILE_BYTES];   // W tile, then X tile
     __shared__ __attribute__((aligned(1024))) unsigned char lds1[2 * TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds2[NS == 4 ? 2 * TILE_BYTES : 16];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds3[NS == 4 ? 2 * TILE_BYTES : 16];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -132,45 +144,82 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+    // Fragment reads are issued as inline asm on plain LDS byte addresses, and waited for with
+    // an explicit lgkmcnt(0) that the fragments pass through ("+v"), for one reason: a read the
+    // compiler can see makes it wait for EVERY outstanding global->LDS load first, which would
+    // undo the prefetch distance of the four-stage pipeline.  Which tile has landed is
+    // tracked by hand with the vmcnt waits at the end of each step.
 #define CUBERT_LOAD_FRAGS(BUF, kk, WF, XF)                                                                  \
     do {                                                                                                    \
+        const int cur = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)(BUF);               \
         _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                      \
-            WF[i] = *reinterpret_cast<const u32x4_t*>((BUF) + (wb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + i * 2048); \
+            asm volatile("ds_read_b128 %0, %1" : "=v"(WF[i])                                                \
+                         : "v"(cur + (wb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + i * 2048));             \
         _Pragma("unroll") for (int j = 0; j < NB; ++j)                                                      \
-            XF[j] = *reinterpret_cast<const u32x4_t*>((BUF) + (xb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + j * 2048); \
+            asm volatile("ds_read_b128 %0, %1" : "=v"(XF[j])                                                \
+                         : "v"(cur + (xb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + j * 2048));             \
+    } while (0)
+#define CUBERT_FENCE_FRAGS(WF, XF)                                                                          \
+    do {                                                                                                    \
+        if constexpr (NB == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(XF[0]));             \
+        if constexpr (NB == 2)                                                                              \
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(WF[1]), "+v"(XF[0]), "+v"(XF[1]));      \
+        if constexpr (NB == 4)                                                                              \
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(WF[1]), "+v"(WF[2]), "+v"(WF[3]),       \
+                         "+v"(XF[0]), "+v"(XF[1]), "+v"(XF[2]), "+v"(XF[3]));                               \
     } while (0)
 
-    // One K step on buffer CUR while the loads for the next step fill NEXT.
+    // One K step on buffer CUR while the loads of the tile NS - 1 steps ahead fill NEXT
+    // (the buffer the previous step computed on; its barrier has released it).
     // The empty asm keeps the compiler from hoisting (and then spilling) every
     // per-k-step address.
 #define CUBERT_K_STEP(CUR, NEXT, kt)                                                                        \
     do {                                                                                                    \
-        CUBERT_ISSUE_TILE(NEXT, (kt) + 1);                                                                  \
+        CUBERT_ISSUE_TILE(NEXT, (kt) + NS - 1);                                                             \
         int wb = woff0, xb = xoff0;                                                                         \
         asm volatile("" : "+v"(wb), "+v"(xb));                                                              \
         u32x4_t wf[2][NB], xf[2][NB];                                                                       \
         CUBERT_LOAD_FRAGS(CUR, 0, wf[0], xf[0]);                                                            \
+        CUBERT_FENCE_FRAGS(wf[0], xf[0]);                                                                   \
         _Pragma("unroll") for (int kk = 0; kk < 4; ++kk) {                                                  \
             if (kk < 3) CUBERT_LOAD_FRAGS(CUR, kk + 1, wf[(kk + 1) & 1], xf[(kk + 1) & 1]);                 \
             _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                  \
                 _Pragma("unroll") for (int j = 0; j < NB; ++j)                                              \
                     mfma_chunk<ELT>(wf[kk & 1][i], xf[kk & 1][j], acc[i][j]);                               \
+            if (kk < 3) CUBERT_FENCE_FRAGS(wf[(kk + 1) & 1], xf[(kk + 1) & 1]);                             \
         }                                                                                                   \
         __builtin_amdgcn_sched_barrier(0);  /* nothing moves across the end of the step */                  \
-        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): my share of NEXT has landed */                     \
-        __syncthreads();                                                                                    \
+        __builtin_amdgcn_s_waitcnt(WAIT_IMM); /* my share of the next step's tile has landed */            \
+        __builtin_amdgcn_s_barrier(); /* bare: a fenced barrier would wait for every load in flight */     \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
     } while (0)
 
     CUBERT_ISSUE_TILE(lds0, kt0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    for (int kt = kt0; kt < KT; kt += 2) {
-        CUBERT_K_STEP(lds0, lds1, kt);
-        CUBERT_K_STEP(lds1, lds0, kt + 1);
+    if constexpr (NS == 4) {
+        CUBERT_ISSUE_TILE(lds1, kt0 + 1);
+        CUBERT_ISSUE_TILE(lds2, kt0 + 2);
+    }
+    __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+    __builtin_amdgcn_s_barrier();
+    if constexpr (NS == 4) {
+        for (int kt = kt0; kt < KT; kt += 4) {
+            CUBERT_K_STEP(lds0, lds3, kt);
+            CUBERT_K_STEP(lds1, lds0, kt + 1);
+            CUBERT_K_STEP(lds2, lds1, kt + 2);
+            CUBERT_K_STEP(lds3, lds2, kt + 3);
+        }
+        // the zero tiles fetched past the end may still be landing in lds0, the epilogue's staging area
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+    } else {
+        for (int kt = kt0; kt < KT; kt += 2) {
+            CUBERT_K_STEP(lds0, lds1, kt);
+            CUBERT_K_STEP(lds1, lds0, kt + 1);
+        }
     }
 #undef CUBERT_ISSUE_TILE
 #undef CUBERT_LOAD_FRAGS
+#undef CUBERT_FENCE_FRAGS
 #undef CUBERT_K_STEP
 
     f32x4_t bias[4 * NB];      // fetched here rather than before the loop: no registers to spare there
