@@ -42,7 +42,7 @@ namespace {
 
 using namespace gemm_detail;
 
-template <int ELT, int OUT, int EPI, int BT>
+template <int ELT, int OUT, int EPI, int BT, int NS>
 __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     constexpr int ES = (ELT == kBF16) ? 2 : 4;       // operand element size
     constexpr int NB = BT / 64;                      // 32x32 blocks per wave and dimension
@@ -52,9 +52,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     constexpr int SBDIV = BT / 16;                   // 16-row groups per sub-block
     constexpr int BK = 128 / ES;                     // K elements per step
 
-    // LDS stages: four for the 64 tile (64 KiB, two workgroups still fit a CU); the 128 tile keeps
-    // two (four would cost it the second resident workgroup), the 256 tile fills the LDS with two.
-    constexpr int NS = (BT == 64) ? 4 : 2;
+    // NS = LDS stages: two, or four for the 64 tile of a launch with few workgroups (64 KiB; with
+    // many workgroups the four resident ones that two stages allow hide the latency better).
+    static_assert(NS == 2 || (NS == 4 && BT == 64), "four stages only fit the 64 tile");
     constexpr int LPT = 2 * GROUPS;                  // loads a wave issues per step
     // s_waitcnt vmcnt(n) with n = the loads of the NS - 2 youngest tiles: the next tile has landed
     constexpr int WAIT_N = LPT * (NS - 2);
@@ -144,29 +144,32 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // Fragment reads are issued as inline asm on plain LDS byte addresses, and waited for with
-    // an explicit lgkmcnt(0) that the fragments pass through ("+v"), for one reason: a read the
-    // compiler can see makes it wait for EVERY outstanding global->LDS load first, which would
-    // undo the prefetch distance of the four-stage pipeline.  Which tile has landed is
-    // tracked by hand with the vmcnt waits at the end of each step.
+    // With four stages the fragment reads are issued as inline asm on plain LDS byte addresses,
+    // and waited for with an explicit lgkmcnt(0) that the fragments pass through ("+v"): a read
+    // the compiler can see makes it wait for EVERY outstanding global->LDS load first, which
+    // would undo the prefetch distance.  Which tile has landed is tracked by hand with the
+    // vmcnt waits at the end of each step.  With two stages every load has landed at the end
+    // of a step anyway and the compiler places the reads and their waits itself.
 #define CUBERT_LOAD_FRAGS(BUF, kk, WF, XF)                                                                  \
     do {                                                                                                    \
-        const int cur = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)(BUF);               \
-        _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                      \
-            asm volatile("ds_read_b128 %0, %1" : "=v"(WF[i])                                                \
-                         : "v"(cur + (wb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + i * 2048));             \
-        _Pragma("unroll") for (int j = 0; j < NB; ++j)                                                      \
-            asm volatile("ds_read_b128 %0, %1" : "=v"(XF[j])                                                \
-                         : "v"(cur + (xb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + j * 2048));             \
+        if constexpr (NS == 4) {                                                                            \
+            const int cur = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)(BUF);           \
+            _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                  \
+                asm volatile("ds_read_b128 %0, %1" : "=v"(WF[i])                                            \
+                             : "v"(cur + (wb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + i * 2048));         \
+            _Pragma("unroll") for (int j = 0; j < NB; ++j)                                                  \
+                asm volatile("ds_read_b128 %0, %1" : "=v"(XF[j])                                            \
+                             : "v"(cur + (xb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + j * 2048));         \
+        } else {                                                                                            \
+            _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                  \
+                WF[i] = *reinterpret_cast<const u32x4_t*>((BUF) + (wb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + i * 2048); \
+            _Pragma("unroll") for (int j = 0; j < NB; ++j)                                                  \
+                XF[j] = *reinterpret_cast<const u32x4_t*>((BUF) + (xb ^ (((kk) & 1) << 5)) + ((kk) >> 1) * SUB + j * 2048); \
+        }                                                                                                   \
     } while (0)
 #define CUBERT_FENCE_FRAGS(WF, XF)                                                                          \
     do {                                                                                                    \
-        if constexpr (NB == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(XF[0]));             \
-        if constexpr (NB == 2)                                                                              \
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(WF[1]), "+v"(XF[0]), "+v"(XF[1]));      \
-        if constexpr (NB == 4)                                                                              \
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(WF[1]), "+v"(WF[2]), "+v"(WF[3]),       \
-                         "+v"(XF[0]), "+v"(XF[1]), "+v"(XF[2]), "+v"(XF[3]));                               \
+        if constexpr (NS == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(WF[0]), "+v"(XF[0]));             \
     } while (0)
 
     // One K step on buffer CUR while the loads of the tile NS - 1 steps ahead fill NEXT
@@ -190,7 +193,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
         }                                                                                                   \
         __builtin_amdgcn_sched_barrier(0);  /* nothing moves across the end of the step */                  \
         __builtin_amdgcn_s_waitcnt(WAIT_IMM); /* my share of the next step's tile has landed */            \
-        __builtin_amdgcn_s_barrier(); /* bare: a fenced barrier would wait for every load in flight */     \
+        if constexpr (NS == 4) __builtin_amdgcn_s_barrier(); /* bare: a fenced one waits for all loads */  \
+        else __syncthreads();                                                                               \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
     } while (0)
 
@@ -200,7 +204,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
         CUBERT_ISSUE_TILE(lds2, kt0 + 2);
     }
     __builtin_amdgcn_s_waitcnt(WAIT_IMM);
-    __builtin_amdgcn_s_barrier();
+    if constexpr (NS == 4) __builtin_amdgcn_s_barrier();
+    else __syncthreads();
     if constexpr (NS == 4) {
         for (int kt = kt0; kt < KT; kt += 4) {
             CUBERT_K_STEP(lds0, lds3, kt);
@@ -223,14 +228,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #undef CUBERT_K_STEP
 
     f32x4_t bias[4 * NB];      // fetched here rather than before the loop: no registers to spare there
-    gemm_load_bias<NB>(p, n0 + wn * (BT / 2), g, bias);
+    constexpr bool SPLITK = EPI == kEpiBias && OUT == kF32;      // the only combination launch_gemm splits
+    gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
     // every wave is past the last step's barrier: the tiles are dead, lds0 is free for staging
-    gemm_epilogue<OUT, EPI, NB>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
+    gemm_epilogue<OUT, EPI, NB, SPLITK>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
 }
 
-template <int ELT, int OUT, int EPI, int BT>
+template <int ELT, int OUT, int EPI, int BT, int NS = 2>
 bool launch_one(const GemmDev& d, hipStream_t stream) {
-    hipLaunchKernelGGL((gemm_kernel<ELT, OUT, EPI, BT>), dim3(d.tiles_n * d.tiles_m, d.splits), dim3(256), 0, stream, d);
+    hipLaunchKernelGGL((gemm_kernel<ELT, OUT, EPI, BT, NS>), dim3(d.tiles_n * d.tiles_m, d.splits), dim3(256), 0, stream, d);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }
@@ -238,7 +244,10 @@ bool launch_one(const GemmDev& d, hipStream_t stream) {
 template <int ELT, int OUT, int EPI>
 bool launch_tile(const GemmDev& d, int bt, hipStream_t stream) {
     switch (bt) {
-        case 64: return launch_one<ELT, OUT, EPI, 64>(d, stream);
+        case 64:
+            // few workgroups: nothing else on the CU hides the memory latency, so prefetch deeper
+            if ((long)d.tiles_n * d.tiles_m * d.splits <= 512) return launch_one<ELT, OUT, EPI, 64, 4>(d, stream);
+            return launch_one<ELT, OUT, EPI, 64>(d, stream);
         case 128: return launch_one<ELT, OUT, EPI, 128>(d, stream);
         case 256: return launch_one<ELT, OUT, EPI, 256>(d, stream);
     }
@@ -262,16 +271,27 @@ bool launch_epi(const GemmDev& d, int epi, int bt, hipStream_t stream) {
 }  // namespace
 
 int gemm_pick_tile(int M, int N, int K, int elt) {
-    // Largest tile that still yields a few workgroups per CU-round; the 256
-    // tile has the best MFMA:LDS ratio, the small ones fill the chip when the
-    // problem is short.  The hand-scheduled bf16 256 kernel runs a tile at about
-    // twice the rate of the general kernel, so it is still the better choice
-    // when its tiles cover well under half of the CUs.
     auto tiles = [&](int bt) { return (long)((M + bt - 1) / bt) * ((N + bt - 1) / bt); };
-    if (tiles(256) >= 256) return 256;
-    if (elt == kBF16 && K % 128 == 0 && tiles(256) >= 160) return 256;
-    if (tiles(128) >= 256) return 128;
-    return 64;
+    auto rounds = [](long wgs, long slots) { return (double)((wgs + slots - 1) / slots); };
+    if (elt != kBF16) {
+        // float32 operands: a 128 tile keeps two workgroups on a CU, which the compiler-scheduled
+        // loop needs more than the larger tile's operand reuse (measured 20 % faster than 256).
+        return tiles(128) >= 512 ? 128 : 64;
+    }
+    // bf16: estimated time = rounds over the chip x time of one workgroup, with per-step costs
+    // measured on MI355X (microseconds): the hand-scheduled 256 tile (one workgroup per CU)
+    // 9 + 0.75 per 32 k; the 128 tile (two per CU) 5 + 1.2 per 64 k; the 64 tile (four per CU)
+    // 4 + 0.9 per 64 k.
+    const double c128 = rounds(tiles(128), 512) * (5.0 + 1.2 * K / 64.0);
+    const double c64 = rounds(tiles(64), 1024) * (4.0 + 0.9 * K / 64.0);
+    double best = c128;
+    int bt = 128;
+    if (c64 < best) { best = c64; bt = 64; }
+    if (K % 128 == 0) {
+        const double c256 = rounds(tiles(256), 256) * (9.0 + 0.75 * K / 32.0);
+        if (c256 <= best) bt = 256;
+    }
+    return bt;
 }
 
 bool launch_gemm(const GemmParams& p, hipStream_t stream) {

@@ -116,17 +116,20 @@ __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, i
 // The bias values a lane needs (4 NB quads) are fetched by gemm_load_bias before the
 // K loop so that their latency is hidden; features past N read the last valid quad
 // (their results are never stored).
-template <int NB>
+template <int NB, bool SPLITK = false>
 __device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int g, f32x4_t (&bias)[4 * NB]) {
 #pragma unroll
     for (int t = 0; t < 4 * NB; ++t) {
         const int n = n_base + 8 * t + 4 * g;
         bias[t] = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
-        if (blockIdx.y != 0) bias[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};     // split K: the bias is added once
+        if constexpr (SPLITK)
+            if (blockIdx.y != 0) bias[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};     // split K: the bias is added once
     }
 }
 
-template <int OUT, int EPI, int NB>
+// SPLITK: the launch may have several workgroups per tile (blockIdx.y = K share), each writing
+// its partial result to its own copy of Y.
+template <int OUT, int EPI, int NB, bool SPLITK = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NB][NB], const f32x4_t (&bias)[4 * NB],
                                               int n_base, int m_base, int l32, int g, unsigned char* scratch) {
     constexpr int OES = (OUT == kBF16) ? 2 : 4;
@@ -208,7 +211,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 // packed bf16 result: the next GEMM's activation operand
                 *reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)) = d;
             } else {
-                *reinterpret_cast<u32x4_t*>(p.Y + (((size_t)blockIdx.y * p.M + mm) * p.N + n) * OES) = d;
+                const size_t part = SPLITK ? (size_t)blockIdx.y * p.M : 0;
+                *reinterpret_cast<u32x4_t*>(p.Y + ((part + mm) * p.N + n) * OES) = d;
             }
         }
     }
