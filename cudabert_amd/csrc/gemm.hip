@@ -37,6 +37,7 @@
 namespace cubert {
 
 bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
+bool launch_gemm_bf16_t256x128(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
 
 namespace {
 
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     constexpr bool SPLITK = EPI == kEpiBias && OUT == kF32;      // the only combination launch_gemm splits
     gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
     // every wave is past the last step's barrier: the tiles are dead, lds0 is free for staging
-    gemm_epilogue<OUT, EPI, NB, SPLITK>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
+    gemm_epilogue<OUT, EPI, NB, NB, SPLITK>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
 }
 
 template <int ELT, int OUT, int EPI, int BT, int NS = 2>
@@ -280,8 +281,10 @@ int gemm_pick_tile(int M, int N, int K, int elt) {
     }
     // bf16: estimated time = rounds over the chip x time of one workgroup, with per-step costs
     // measured on MI355X (microseconds): the hand-scheduled 256 tile (one workgroup per CU)
-    // 9 + 0.75 per 32 k; the 128 tile (two per CU) 5 + 1.2 per 64 k; the 64 tile (four per CU)
-    // 4 + 0.9 per 64 k.
+    // 9 + 0.75 per 32 k; the hand-scheduled 256 x 128 tile (two per CU, which overlap instead of
+    // running in rounds) 4.5 + 0.98 per 32 k (1.06 for K > 1536, where its shorter prefetch
+    // distance shows); the 128 tile (two per CU) 5 + 1.2 per 64 k; the
+    // 64 tile (four per CU) 4 + 0.9 per 64 k.
     const double c128 = rounds(tiles(128), 512) * (5.0 + 1.2 * K / 64.0);
     const double c64 = rounds(tiles(64), 1024) * (4.0 + 0.9 * K / 64.0);
     double best = c128;
@@ -289,7 +292,12 @@ int gemm_pick_tile(int M, int N, int K, int elt) {
     if (c64 < best) { best = c64; bt = 64; }
     if (K % 128 == 0) {
         const double c256 = rounds(tiles(256), 256) * (9.0 + 0.75 * K / 32.0);
-        if (c256 <= best) bt = 256;
+        if (c256 <= best) { best = c256; bt = 256; }
+    }
+    {
+        const double wgs = (double)((M + 127) / 128) * ((N + 255) / 256);
+        const double c384 = (wgs > 512.0 ? wgs / 512.0 : 1.0) * (4.5 + (K > 1536 ? 1.06 : 0.98) * K / 32.0);
+        if (c384 < best) bt = kTile256x128;
     }
     return bt;
 }
@@ -355,6 +363,12 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     }
     int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
     if (d.splits > 1 && bt == 256 && !p.tile) bt = 128;      // the hand-scheduled kernel does not split
+    if (bt == kTile256x128) {
+        if (p.elt != kBF16 || d.splits != 1) { set_error("gemm: the 256x128 tile is bf16 only and does not split K"); return false; }
+        d.tiles_n = (p.N + 255) / 256;
+        d.tiles_m = (p.M + 127) / 128;
+        return launch_gemm_bf16_t256x128(d, out, epi, stream);
+    }
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
     if (p.elt == kBF16) {

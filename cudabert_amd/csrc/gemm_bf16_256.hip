@@ -88,7 +88,89 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
 
     // Stages 0 and 1 were last read two barriers ago; the tail of the loop only reads stages
     // 2 and 3, so the first 64 KiB are free for the epilogue's staging while slower waves finish.
-    gemm_epilogue<OUT, EPI, 4>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
+    gemm_epilogue<OUT, EPI, 4, 4>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
+}
+
+// ---------------------------------------------------------------------------
+// 256 features x 128 tokens per workgroup, two workgroups per CU (loop:
+// gemm_bf16_256x128_loop.inc, "half" mode of gen_gemm_asm.py).  A wave owns 128 x 64
+// = 4 x 2 accumulator blocks and stays below 128 VGPRs, so each SIMD holds one wave of
+// each workgroup: the prologue, epilogue and launch gap of one workgroup overlap the
+// other's main loop.  Costs 1.5x the LDS fragment traffic per flop of the 256 x 256 tile.
+#define CUBERT_ACC_OPERANDS_H                                                                            \
+    [c00] "=&a"(acc[0][0]), [c01] "=&a"(acc[0][1]), [c10] "=&a"(acc[1][0]), [c11] "=&a"(acc[1][1]),         \
+    [c20] "=&a"(acc[2][0]), [c21] "=&a"(acc[2][1]), [c30] "=&a"(acc[3][0]), [c31] "=&a"(acc[3][1])
+
+template <int OUT, int EPI>
+__global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDev p) {
+    // Three stages of 24 KiB: W tile (256 rows x 64 B) at +0, X tile (128 rows x 64 B) at +0x4000.
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[3 * 24576];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave >> 1, wm = wave & 1;
+    const int l32 = lane & 31, g = lane >> 5;
+
+    int tile_n, tile_m;
+    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, &tile_n, &tile_m);
+    const int n0 = tile_n * 256, m0 = tile_m * 128;
+
+    const unsigned long long wa = reinterpret_cast<unsigned long long>(p.W);
+    const unsigned long long xa = reinterpret_cast<unsigned long long>(p.X);
+    const unsigned wsize = p.w_packed ? (unsigned)packed_bytes(p.N, (size_t)p.K * 2) : (unsigned)((size_t)p.N * p.K * 2);
+    const unsigned xsize = p.x_packed ? (unsigned)packed_bytes(p.M, (size_t)p.K * 2)
+                                      : (unsigned)((((size_t)p.M - 1) * p.ldx + p.K) * 2);
+    const u32x4_t wres = {(unsigned)wa, (unsigned)(wa >> 32) & 0xffffu, wsize, 0x00020000u};
+    const u32x4_t xres = {(unsigned)xa, (unsigned)(xa >> 32) & 0xffffu, xsize, 0x00020000u};
+    const int w_rowb = p.K * 2, x_rowb = p.ldx * 2;
+    const int KB = p.K * 2 / 64;
+    // One load moves 16 rows x 64 bytes.  Wave w moves the W row groups w, w+4, w+8, w+12 and the
+    // X row groups w, w+4 of each tile (see the 256 x 256 kernel for the chunk choice `dc`).
+    const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
+    const int w_v0 = p.w_packed ? (tile_n * KB * 16384 + wave * 1024 + lane * 16)
+                                : ((n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4));
+    const int x_v0 = p.x_packed ? ((m0 >> 8) * KB * 16384 + (m0 & 255) * 64 + wave * 1024 + lane * 16)
+                                : ((m0 + 16 * wave + (lane >> 2)) * x_rowb + (dc << 4));
+    const int w64 = p.w_packed ? 4096 : 64 * w_rowb, x64 = p.x_packed ? 4096 : 64 * x_rowb;
+    const int wkstep = p.w_packed ? 16384 : 64, xkstep = p.x_packed ? 16384 : 64;
+    const int lds_base = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+    const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
+    const int wb = lds_base + (wn * 128 + l32) * 64 + ((g ^ sw) << 4);
+    const int xb = lds_base + (wm * 64 + l32) * 64 + ((g ^ sw) << 4);       // + 0x4000 is in the read offsets
+    const int m0b = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
+    const int ht = p.K / 32;
+
+    f32x16_t acc[4][2];       // zeroed inside the asm block
+
+    asm volatile(
+#include "gemm_bf16_256x128_loop.inc"
+        : CUBERT_ACC_OPERANDS_H
+        : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
+          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep)
+        : "memory", "scc", "s92", "s93", "s94", "s96", "s97", "s98", "v64", "v65", "v66", "v67", "v68", "v69",
+          CUBERT_V10(7), CUBERT_V10(8), CUBERT_V10(9), CUBERT_V10(10), CUBERT_V10(11), "v120", "v121", "v122",
+          "v123", "v124", "v125");
+
+    // The block ends with all loads landed and a barrier: the whole LDS is free for staging.
+    f32x4_t bias[16];
+    gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
+    gemm_epilogue<OUT, EPI, 4, 2>(p, acc, bias, n0 + wn * 128, m0 + wm * 64, l32, g, lds + wave * 16384);
+}
+
+template <int OUT>
+bool launch_epi_half(const GemmDev& d, int epi, hipStream_t stream) {
+    const dim3 grid(d.tiles_n * d.tiles_m), block(256);
+    switch (epi) {
+        case kEpiBias: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBias>), grid, block, 0, stream, d); break;
+        case kEpiBiasGelu: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBiasGelu>), grid, block, 0, stream, d); break;
+        case kEpiBiasTanh: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBiasTanh>), grid, block, 0, stream, d); break;
+        case kEpiQKV: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiQKV>), grid, block, 0, stream, d); break;
+        case kEpiQKVMap: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiQKVMap>), grid, block, 0, stream, d); break;
+        default: set_error("gemm: unknown epilogue"); return false;
+    }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
 }
 
 template <int OUT>
@@ -112,6 +194,13 @@ bool launch_epi(const GemmDev& d, int epi, hipStream_t stream) {
 bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream) {
     if (d.K % 128 != 0 || d.K < 128) { set_error("gemm: the 256 tile needs K to be a multiple of 128"); return false; }
     return out_elt == kBF16 ? launch_epi<kBF16>(d, epilogue, stream) : launch_epi<kF32>(d, epilogue, stream);
+}
+
+
+// 256 x 128 tile: d.tiles_n for 256 features, d.tiles_m for 128 tokens; d.K % 32 == 0, K >= 64.
+bool launch_gemm_bf16_t256x128(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream) {
+    if (d.K % 32 != 0 || d.K < 64) { set_error("gemm: the 256x128 tile needs K to be a multiple of 32, at least 64"); return false; }
+    return out_elt == kBF16 ? launch_epi_half<kBF16>(d, epilogue, stream) : launch_epi_half<kF32>(d, epilogue, stream);
 }
 
 }  // namespace cubert

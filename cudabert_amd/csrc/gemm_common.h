@@ -116,10 +116,10 @@ __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, i
 // The bias values a lane needs (4 NB quads) are fetched by gemm_load_bias before the
 // K loop so that their latency is hidden; features past N read the last valid quad
 // (their results are never stored).
-template <int NB, bool SPLITK = false>
-__device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int g, f32x4_t (&bias)[4 * NB]) {
+template <int NBI, bool SPLITK = false>
+__device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int g, f32x4_t (&bias)[4 * NBI]) {
 #pragma unroll
-    for (int t = 0; t < 4 * NB; ++t) {
+    for (int t = 0; t < 4 * NBI; ++t) {
         const int n = n_base + 8 * t + 4 * g;
         bias[t] = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
         if constexpr (SPLITK)
@@ -129,11 +129,12 @@ __device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int
 
 // SPLITK: the launch may have several workgroups per tile (blockIdx.y = K share), each writing
 // its partial result to its own copy of Y.
-template <int OUT, int EPI, int NB, bool SPLITK = false>
-__device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NB][NB], const f32x4_t (&bias)[4 * NB],
+// The wave's quadrant is NBI x NBJ accumulator blocks (features x tokens).
+template <int OUT, int EPI, int NBI, int NBJ, bool SPLITK = false>
+__device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NBI][NBJ], const f32x4_t (&bias)[4 * NBI],
                                               int n_base, int m_base, int l32, int g, unsigned char* scratch) {
     constexpr int OES = (OUT == kBF16) ? 2 : 4;
-    constexpr int RB = 32 * NB * OES;       // bytes per token row of the staging block
+    constexpr int RB = 32 * NBI * OES;      // bytes per token row of the staging block
     constexpr int CH = RB / 16;             // 16-byte chunks per row
     constexpr int RPI = 64 / CH;            // rows one store instruction covers
     constexpr int EPC = 16 / OES;           // elements per chunk
@@ -141,16 +142,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
     const int rrow = lane / CH, rc = lane % CH;
     // compact rows: the token of this lane's row in every block row, fetched together up front;
     // the read-out phase takes a row's token from the lane that owns it
-    int tokj[NB];
+    int tokj[NBJ];
     if constexpr (EPI == kEpiQKVMap) {
 #pragma unroll
-        for (int j = 0; j < NB; ++j) {
+        for (int j = 0; j < NBJ; ++j) {
             const int m = m_base + 32 * j + l32;
             tokj[j] = p.rowmap[m < p.M ? m : p.M - 1];
         }
     }
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
+    for (int j = 0; j < NBJ; ++j) {
         unsigned char* buf = scratch + ((OES == 2 && (j & 1)) ? 32 * RB : 0);
         const int m = m_base + 32 * j + l32;
         int bidx = 0, sidx = 0;
@@ -161,7 +162,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             sidx = tok - bidx * p.S;
         }
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
+        for (int i = 0; i < NBI; ++i) {
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
                 const int fq = 32 * i + 8 * qd + 4 * g;          // feature within the quadrant

@@ -369,8 +369,143 @@ def main_staged():
         print('"%s\\n"' % ln)
 
 
+
+
+
+# ---------------------------------------------------------------------------
+# 256 x 128 macro tile, two workgroups per CU ("half" mode):
+#     python gen_gemm_asm.py half > gemm_bf16_256x128_loop.inc
+#
+# A wave owns 128 features x 64 tokens = 4 x 2 accumulator blocks (128 AGPRs) and
+# stays below 128 VGPRs, so a SIMD holds two waves of two different workgroups:
+# while one workgroup is in its prologue or epilogue the other one's main loop
+# has the matrix pipe.  Three LDS stages of 24 KiB (W tile 256 rows x 64 B at +0,
+# X tile 128 rows x 64 B at +0x4000); the tile of half-step h lives in stage
+# h % 3 and the loads of tile h+2 are issued during half-step h.  The loop body
+# is ONE half-step; the stage rotates through scalar byte offsets, so any number
+# of half-steps works and there is no separate tail:
+#   s92  stage offset of the tile being multiplied      (0, 0x6000, 0xC000)
+#   s93  stage offset of the tile being fetched
+#   s94  M0 base (LDS base + wave * 1024)   s96 / s98  K byte offsets   s97  counter
+#   v112..v115  fragment row addresses in stage 0: W k-phase 0, W k-phase 1, X k-phase 0, X k-phase 1
+#   v122..v125  the same for the current stage      v116..v119 / v120..v121  W / X lane offsets
+#   v64..v79 / v80..v87  W / X fragments, set A      v88..v103 / v104..v111  set B
+# A half-step: 6 reads of k-phase 0 (set A), 8 MFMAs on A with the 6 reads of k-phase 1
+# (set B) and the 6 global->LDS loads behind them, 8 MFMAs on B, vmcnt(6) (everything but
+# the loads just issued, i.e. tile h+1, has landed), barrier.  The reads at the top are
+# not hidden inside the wave; the other workgroup's wave on the SIMD covers them.  Loads
+# issued for tiles past the end of K fetch valid memory or zeros and are never used; the
+# block ends with vmcnt(0) and a barrier so that nothing lands in the LDS afterwards.
+H_WA, H_XA, H_WB, H_XB = 64, 80, 88, 104
+H_BASE, H_CUR = 112, 122
+H_WVOFF, H_XVOFF = 116, 120
+H_STAGE = 0x6000
+
+
+def main_half():
+    e = Emitter()
+    e.emit("; ======== setup ========")
+    e.emit("v_mov_b32 v%d, %%[wb]" % (H_BASE + 0))
+    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (H_BASE + 1))
+    e.emit("v_mov_b32 v%d, %%[xb]" % (H_BASE + 2))
+    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (H_BASE + 3))
+    e.emit("v_mov_b32 v%d, %%[wv0]" % H_WVOFF)
+    e.emit("v_mov_b32 v%d, %%[xv0]" % H_XVOFF)
+    for i in range(1, 4):
+        e.emit("v_add_u32 v%d, %%[w64], v%d" % (H_WVOFF + i, H_WVOFF + i - 1))
+    e.emit("v_add_u32 v%d, %%[x64], v%d" % (H_XVOFF + 1, H_XVOFF))
+    for r in range(4):
+        e.emit("v_mov_b32 v%d, 0" % (H_WA + r))
+    e.emit("s_nop 7")      # VALU result -> MFMA source operand
+    for i in range(4):
+        for j in range(2):
+            e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, 0" % (i, j, vreg4(H_WA), vreg4(H_WA)))
+    e.emit("s_mov_b32 s94, %[m0b]")
+    e.emit("s_mov_b32 s92, 0")
+    e.emit("s_mov_b32 s93, 0")
+    e.emit("s_mov_b32 s96, 0")
+    e.emit("s_mov_b32 s98, 0")
+
+    def dma(k):
+        """k-th of the wave's six loads of the tile at stage offset s93: (M0 update, load)."""
+        m0 = "s_add_u32 m0, s94, s93" if k == 0 else "s_add_u32 m0, m0, 0x1000"
+        if k < 4:
+            ld = "buffer_load_dwordx4 v%d, %%[wres], s96 offen lds" % (H_WVOFF + k)
+        else:
+            ld = "buffer_load_dwordx4 v%d, %%[xres], s98 offen lds" % (H_XVOFF + k - 4)
+        return m0, ld
+
+    def rotate(reg):
+        e.emit("s_add_u32 s%d, s%d, 0x%x" % (reg, reg, H_STAGE))
+        e.emit("s_cmp_eq_u32 s%d, 0x%x" % (reg, 3 * H_STAGE))
+        e.emit("s_cselect_b32 s%d, 0, s%d" % (reg, reg))
+
+    e.emit("; ======== prologue: tiles 0, 1 -> stages 0, 1 ========")
+    for t in range(2):
+        for k in range(6):
+            m0, ld = dma(k)
+            e.emit(m0)
+            e.emit("s_nop 0")
+            e.emit(ld)
+        rotate(93)
+        advance_k(e)
+    e.emit("s_waitcnt vmcnt(6)")           # tile 0 has landed
+    e.emit("s_barrier")
+    e.emit("s_mov_b32 s97, 0")
+    e.emit("L_loop_%=:")
+    e.forget_bound()
+    for r in range(4):
+        e.emit("v_add_u32 v%d, s92, v%d" % (H_CUR + r, H_BASE + r))
+
+    def reads(kk, wset, xset):
+        out = [(wset + 4 * b, H_CUR + kk, b * 2048) for b in range(4)]
+        out += [(xset + 4 * b, H_CUR + 2 + kk, 0x4000 + b * 2048) for b in range(2)]
+        # first the pair the first MFMA needs
+        return [out[0], out[4], out[5], out[1], out[2], out[3]]
+
+    for r in reads(0, H_WA, H_XA):
+        e.read(*r)
+    pending = reads(1, H_WB, H_XB)
+    n_dma = 0
+    for kk in range(2):
+        wset, xset = (H_WA, H_XA) if kk == 0 else (H_WB, H_XB)
+        m = 0
+        for i in range(4):
+            for j in range(2):
+                e.need(wset + 4 * i, xset + 4 * j)
+                gm = 8 * kk + m
+                d = n_dma if (gm % 2 == 0 and n_dma < 6) else None
+                if d is not None:
+                    e.emit(dma(d)[0])
+                e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %
+                       (i, j, vreg4(wset + 4 * i), vreg4(xset + 4 * j), i, j))
+                if d is not None:
+                    e.emit(dma(d)[1])
+                    n_dma += 1
+                if kk == 0 and m < len(pending):
+                    e.read(*pending[m])
+                m += 1
+    assert n_dma == 6
+    rotate(92)
+    rotate(93)
+    advance_k(e)
+    e.emit("s_waitcnt vmcnt(6)")
+    e.emit("s_barrier")
+    e.emit("s_add_u32 s97, s97, 1")
+    e.emit("s_cmp_lt_u32 s97, %[ht]")
+    e.emit("s_cbranch_scc1 L_loop_%=")
+    e.emit("s_waitcnt vmcnt(0)")
+    e.emit("s_barrier")
+    print("// Generated by gen_gemm_asm.py half -- do not edit.")
+    for ln in e.lines:
+        print('"%s\\n"' % ln)
+
+
 if __name__ == "__main__":
-    if os.environ.get("CUBERT_GEMM_MODE", "dma") == "staged":
+    import sys
+    if len(sys.argv) > 1 and sys.argv[1] == "half":
+        main_half()
+    elif os.environ.get("CUBERT_GEMM_MODE", "dma") == "staged":
         main_staged()
     else:
         main()

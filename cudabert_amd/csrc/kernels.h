@@ -34,6 +34,8 @@ struct Compact {
     int rows = 0;
 };
 
+constexpr int kTile256x128 = 384;     // GemmParams::tile value of the 256 features x 128 tokens kernel
+
 struct GemmParams {
     const void* X = nullptr;
     const void* W = nullptr;
@@ -52,7 +54,7 @@ struct GemmParams {
     void* vt = nullptr;
     int S = 0, Sp = 0, heads = 0;
     const int* rowmap = nullptr;   // kEpiQKV on compact rows: row m is token rowmap[m] = b * S + s
-    int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile)
+    int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile) or kTile256x128
     // Split K (kEpiBias, float32 Y): `splits` workgroups share a tile, each reduces its share of K and
     // writes its partial result to Y + z * M * N; the bias goes into partial 0.  The consumer adds
     // them up (launch_add_layernorm's y_parts).  Y must hold splits * M * N floats.

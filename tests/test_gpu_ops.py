@@ -76,11 +76,13 @@ def gelu64(x):
 
 
 @pytest.mark.parametrize("elt", [F32, BF16])
-@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("tile", [64, 128, 256, 384])          # 384: the 256 x 128 two-per-CU kernel (bf16)
 @pytest.mark.parametrize("M,N,K,epi", [(200, 128, 128, 0), (333, 384, 256, 1), (512, 1024, 1024, 0),
-                                       (77, 512, 512, 2), (1000, 768, 3072, 0)])
+                                       (77, 512, 512, 2), (1000, 768, 3072, 0), (130, 256, 64, 0)])
 def test_gemm(pb, elt, tile, M, N, K, epi):
     print("gemm", elt, tile, M, N, K, epi, flush=True)
+    if tile == 384 and elt == F32:
+        pytest.skip("the 256 x 128 kernel is bf16 only")
     rng = np.random.default_rng(M * 7 + N + K + epi)
     X = rng.standard_normal((M, K)).astype(np.float32)
     W = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
@@ -135,9 +137,12 @@ def test_gemm_rejects_bad_shapes(pb):
 
 
 @pytest.mark.parametrize("elt", [F32, BF16])
-@pytest.mark.parametrize("B,S,heads,tile", [(3, 33, 2, 64), (2, 200, 4, 128), (5, 128, 12, 256)])
+@pytest.mark.parametrize("B,S,heads,tile", [(3, 33, 2, 64), (2, 200, 4, 128), (5, 128, 12, 256), (2, 200, 4, 384),
+                                            (5, 128, 12, 384)])
 def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile):
     print("qkv", elt, B, S, heads, tile, flush=True)
+    if tile == 384 and elt == F32:
+        pytest.skip("the 256 x 128 kernel is bf16 only")
     rng = np.random.default_rng(B + S)
     H = heads * 64
     Sp = (S + 31) // 32 * 32
@@ -299,7 +304,7 @@ def test_mask_softmax(pb, elt, B, R, S):
     assert (got[np.broadcast_to(mask[:, None, :] == 0, got.shape)] == 0).all()
 
 
-@pytest.mark.parametrize("tile,flags_extra", [(64, 0), (128, 0), (256, 0), (256, 8)])
+@pytest.mark.parametrize("tile,flags_extra", [(64, 0), (128, 0), (256, 0), (256, 8), (384, 0)])
 @pytest.mark.parametrize("M,N,K,epi,xp,wp,yp", [(200, 128, 128, 0, 1, 1, 0), (333, 384, 256, 1, 1, 1, 1), (512, 1024, 1024, 0, 1, 0, 0),
                                                (700, 512, 512, 0, 0, 1, 1), (1000, 768, 3072, 0, 1, 1, 0)])
 def test_gemm_packed_operands(pb, tile, flags_extra, M, N, K, epi, xp, wp, yp):
