@@ -66,8 +66,8 @@ def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
     k_ms = e0.elapsed_time(e1) / launches
     flops_per_launch = 2.0 * N * H * I
     achieved = flops_per_launch / k_ms / 1e9
-    roofline = {"bound": "mfma", "kernel": "gemm_kernel<%s, bias+GELU, tile 256> (FFN-in %dx%dx%d)" %
-                (precision, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[precision],
+    kname = "gemm_bf16_t256x128_kernel<bf16, bias+GELU>" if precision == "bf16" else "gemm_kernel<f32, f32, bias+GELU, 128>"
+    roofline = {"bound": "mfma", "kernel": "%s (FFN-in %dx%dx%d, tile chosen by the library)" % (kname, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[precision],
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[precision], 4),
                 "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch,
                 "traffic": MEASURED_TRAFFIC.get((precision, N, I, H))}

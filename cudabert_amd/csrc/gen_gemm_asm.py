@@ -390,10 +390,11 @@ def main_staged():
 #   v112..v115  fragment row addresses in stage 0: W k-phase 0, W k-phase 1, X k-phase 0, X k-phase 1
 #   v122..v125  the same for the current stage      v116..v119 / v120..v121  W / X lane offsets
 #   v64..v79 / v80..v87  W / X fragments, set A      v88..v103 / v104..v111  set B
-# A half-step: 6 reads of k-phase 0 (set A), 8 MFMAs on A with the 6 reads of k-phase 1
-# (set B) and the 6 global->LDS loads behind them, 8 MFMAs on B, vmcnt(6) (everything but
-# the loads just issued, i.e. tile h+1, has landed), barrier.  The reads at the top are
-# not hidden inside the wave; the other workgroup's wave on the SIMD covers them.  Loads
+# A half-step, skewed by one k-phase so that no fragment read is waited for right after
+# issue: 6 reads of this tile's k-phase 0 (set A); 8 MFMAs on set B = the previous tile's
+# k-phase 1, read a half-step ago; 8 MFMAs on A with the 6 reads of this tile's k-phase 1
+# (into B) behind them; the 6 global->LDS loads of tile h+2 spread behind the MFMAs;
+# vmcnt(6) (everything but the loads just issued, i.e. tile h+1, has landed); barrier.  Loads
 # issued for tiles past the end of K fetch valid memory or zeros and are never used; the
 # block ends with vmcnt(0) and a barrier so that nothing lands in the LDS afterwards.
 H_WA, H_XA, H_WB, H_XB = 64, 80, 88, 104
@@ -451,11 +452,6 @@ def main_half():
         advance_k(e)
     e.emit("s_waitcnt vmcnt(6)")           # tile 0 has landed
     e.emit("s_barrier")
-    e.emit("s_mov_b32 s97, 0")
-    e.emit("L_loop_%=:")
-    e.forget_bound()
-    for r in range(4):
-        e.emit("v_add_u32 v%d, s92, v%d" % (H_CUR + r, H_BASE + r))
 
     def reads(kk, wset, xset):
         out = [(wset + 4 * b, H_CUR + kk, b * 2048) for b in range(4)]
@@ -463,18 +459,20 @@ def main_half():
         # first the pair the first MFMA needs
         return [out[0], out[4], out[5], out[1], out[2], out[3]]
 
-    for r in reads(0, H_WA, H_XA):
-        e.read(*r)
-    pending = reads(1, H_WB, H_XB)
-    n_dma = 0
-    for kk in range(2):
-        wset, xset = (H_WA, H_XA) if kk == 0 else (H_WB, H_XB)
+    def cur_addresses():
+        for r in range(4):
+            e.emit("v_add_u32 v%d, s92, v%d" % (H_CUR + r, H_BASE + r))
+
+    def mfmas(wset, xset, tracked, pending, dma_from):
+        """Eight MFMAs on one fragment set; `pending` LDS reads and the DMA loads
+        dma_from, dma_from + 1, dma_from + 2 go behind them."""
+        n_dma = 0
         m = 0
         for i in range(4):
             for j in range(2):
-                e.need(wset + 4 * i, xset + 4 * j)
-                gm = 8 * kk + m
-                d = n_dma if (gm % 2 == 0 and n_dma < 6) else None
+                if tracked:
+                    e.need(wset + 4 * i, xset + 4 * j)
+                d = dma_from + n_dma if (dma_from is not None and m % 2 == 0 and n_dma < 3) else None
                 if d is not None:
                     e.emit(dma(d)[0])
                 e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %
@@ -482,18 +480,53 @@ def main_half():
                 if d is not None:
                     e.emit(dma(d)[1])
                     n_dma += 1
-                if kk == 0 and m < len(pending):
+                if m < len(pending):
                     e.read(*pending[m])
                 m += 1
-    assert n_dma == 6
-    rotate(92)
-    rotate(93)
-    advance_k(e)
-    e.emit("s_waitcnt vmcnt(6)")
-    e.emit("s_barrier")
+
+    def end_of_half_step():
+        rotate(92)
+        rotate(93)
+        advance_k(e)
+        # vmcnt(6): everything but the loads just issued, i.e. the next tile, has landed.
+        # lgkmcnt(0): my reads of this tile are done before anybody may overwrite its stage.
+        e.emit("s_waitcnt vmcnt(6) lgkmcnt(0)")
+        e.emit("s_barrier")
+
+    # The pipeline is skewed by one k-phase: a half-step starts by reading its tile's k-phase-0
+    # fragments (set A) and multiplies the PREVIOUS tile's k-phase 1 (set B, read a half-step
+    # ago) while they arrive; then k-phase 0 on set A while k-phase 1 is read into set B.
+    e.emit("; ======== half-step 0: no previous tile ========")
+    cur_addresses()
+    for r in reads(0, H_WA, H_XA):
+        e.read(*r)
+    mfmas(H_WA, H_XA, True, reads(1, H_WB, H_XB), 0)
+    # the three remaining loads of tile 2 without MFMAs to hide behind
+    for k in range(3, 6):
+        e.emit(dma(k)[0])
+        e.emit("s_nop 0")
+        e.emit(dma(k)[1])
+    end_of_half_step()
+    e.emit("s_mov_b32 s97, 1")
+    e.emit("s_cmp_ge_u32 s97, %[ht]")
+    e.emit("s_cbranch_scc1 L_last_%=")
+    e.emit("L_loop_%=:")
+    cur_addresses()
+    for r in reads(0, H_WA, H_XA):
+        e.read(*r)
+    e.emit("s_waitcnt lgkmcnt(6)")         # set B (read during the previous half-step) is complete
+    e.forget_bound()
+    e.guaranteed = 6
+    mfmas(H_WB, H_XB, False, [], 0)
+    mfmas(H_WA, H_XA, True, reads(1, H_WB, H_XB), 3)
+    end_of_half_step()
     e.emit("s_add_u32 s97, s97, 1")
     e.emit("s_cmp_lt_u32 s97, %[ht]")
     e.emit("s_cbranch_scc1 L_loop_%=")
+    e.emit("L_last_%=:")
+    e.emit("s_waitcnt lgkmcnt(0)")
+    e.emit("; ======== k-phase 1 of the last tile ========")
+    mfmas(H_WB, H_XB, False, [], None)
     e.emit("s_waitcnt vmcnt(0)")
     e.emit("s_barrier")
     print("// Generated by gen_gemm_asm.py half -- do not edit.")
