@@ -1,8 +1,11 @@
 #!/usr/bin/env python3
-"""Generates gemm_bf16_256_loop.inc: the hand-scheduled main loop (gfx950 ISA,
-as one inline-asm string) of the 256x256 bf16 GEMM macro tile.
+"""Generates the hand-scheduled main loops (gfx950 ISA, each one inline-asm
+string) of the bf16 GEMM macro tiles:
 
-    python gen_gemm_asm.py > gemm_bf16_256_loop.inc
+    python gen_gemm_asm.py      > gemm_bf16_256_loop.inc        # 256 x 256, one workgroup per CU
+    python gen_gemm_asm.py half > gemm_bf16_256x128_loop.inc    # 256 x 128, two per CU (end of file)
+
+The rest of this comment describes the 256 x 256 loop.
 
 Why hand-scheduled: with 256 accumulator registers per lane a SIMD holds one
 wave, so nothing but instruction order hides LDS and memory latency.
@@ -37,11 +40,6 @@ in slot c ^ (((r >> 1) ^ (r >> 3)) & 3), which spreads the fragment reads of any
 16 rows (64 lanes x 16 B) to M0 + 16 * lane; the swizzle is applied on the
 global side (which chunk a lane fetches).
 """
-import os
-
-# Ablation switches for timing experiments only (they break the result).
-ABL = set(os.environ.get("CUBERT_GEMM_ABLATE", "").split(","))
-
 WA, XA, WB, XB = 192, 208, 224, 240
 ADDR = 176            # + 4 * bank + {0: W kk0, 1: W kk1, 2: X kk0, 3: X kk1}
 W_VOFF, X_VOFF = 184, 188
@@ -60,12 +58,6 @@ class Emitter:
         self.guaranteed = None     # an upper bound on outstanding LDS reads already waited for
 
     def emit(self, text):
-        if "nodma" in ABL and text.startswith("buffer_load_dwordx4"):
-            return
-        if "noread" in ABL and text.startswith("ds_read"):
-            return
-        if "nomfma" in ABL and text.startswith("v_mfma"):
-            return
         self.lines.append(text)
 
     def read(self, dst, addr_reg, offset):
@@ -81,21 +73,6 @@ class Emitter:
         (LDS reads return in order)."""
         newest = max(self.index[r] for r in regs)
         allowed = self.issued - 1 - newest
-        if self.guaranteed is None or allowed < self.guaranteed:
-            self.emit("s_waitcnt lgkmcnt(%d)" % min(allowed, 15))
-            self.guaranteed = allowed
-
-    def write(self, data, addr_reg, offset):
-        assert 0 <= offset < 65536
-        self.emit("ds_write_b128 v%d, %s offset:%d" % (addr_reg, vreg4(data), offset))
-        self.last_write = self.issued
-        self.issued += 1
-        if self.guaranteed is not None:
-            self.guaranteed += 1
-
-    def need_writes(self):
-        """s_waitcnt so that every LDS write issued so far has completed."""
-        allowed = self.issued - 1 - self.last_write
         if self.guaranteed is None or allowed < self.guaranteed:
             self.emit("s_waitcnt lgkmcnt(%d)" % min(allowed, 15))
             self.guaranteed = allowed
@@ -131,7 +108,7 @@ def dma_instrs(stage):
     return out
 
 
-DMA_EVERY = int(os.environ.get("CUBERT_GEMM_DMA_EVERY", "2"))   # one global->LDS load behind every n-th MFMA
+DMA_EVERY = 2         # one global->LDS load behind every second MFMA
 
 
 def half_step(e, stage, dma, prefetch_next, vmcnt, barrier):
@@ -234,142 +211,6 @@ def main():
     print("// Generated by gen_gemm_asm.py -- do not edit.")
     for ln in e.lines:
         print('"%s\\n"' % ln)
-
-
-# ---------------------------------------------------------------------------
-# Register-staged variant: global -> VGPR (buffer_load_dwordx4), one half-step
-# later VGPR -> LDS (ds_write_b128).  The global->LDS path above keeps the LDS
-# busy for as long as the data trickles in from the texture unit; staging
-# through registers writes a tile in a quarter of that time, which leaves the
-# LDS to the fragment reads.
-#   half-step h:  phase 0  fragment reads (tile h, k-phase 1) behind MFMA 0..7,
-#                          wait for the loads of tile h+2, write it to stage (h+2)%4
-#                          behind MFMA 8..15 (register set h % 2)
-#                 phase 1  fragment reads (tile h+1, k-phase 0) behind MFMA 0..7,
-#                          global loads of tile h+4 into register set h % 2 behind MFMA 8..15
-#                 end      wait for the LDS writes, s_barrier
-LD_REGS = [100, 132]      # two sets of eight 4-register destinations
-LDSW = 170                # v170: my LDS write address in stages 0/1, v171: the same + 65536
-
-
-def load_instrs(regset):
-    out = []
-    for k in range(8):
-        dst = vreg4(LD_REGS[regset] + 4 * k)
-        if k < 4:
-            out.append("buffer_load_dwordx4 %s, v%d, %%[wres], s96 offen" % (dst, W_VOFF + k))
-        else:
-            out.append("buffer_load_dwordx4 %s, v%d, %%[xres], s98 offen" % (dst, X_VOFF + k - 4))
-    return out
-
-
-def write_instrs(regset, stage):
-    bank, half = stage >> 1, stage & 1
-    return [(LD_REGS[regset] + 4 * k, LDSW + bank, half * 32768 + (0 if k < 4 else 16384) + (k % 4) * 4096)
-            for k in range(8)]
-
-
-def half_step_staged(e, h, write_vmcnt, do_load, prefetch_next, barrier):
-    """write_vmcnt: None (nothing to write) or the vmcnt that guarantees tile h+2 has arrived."""
-    stage = h % NSTAGE
-    e.emit("; ---- half-step on stage %d (register-staged)" % stage)
-    writes = write_instrs(h % 2, (stage + 2) % NSTAGE) if write_vmcnt is not None else []
-    loads = load_instrs(h % 2) if do_load else []
-    for kk in range(2):
-        wset, xset = (WA, XA) if kk == 0 else (WB, XB)
-        if kk == 0:
-            pending = frag_reads(stage, 1, WB, XB)
-        else:
-            pending = frag_reads((stage + 1) % NSTAGE, 0, WA, XA) if prefetch_next else []
-        m = 0
-        for i in range(4):
-            for j in range(4):
-                e.need(wset + 4 * i, xset + 4 * j)
-                if kk == 0 and m == 8 and writes:
-                    e.emit("s_waitcnt vmcnt(%d)" % write_vmcnt)
-                e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %
-                       (i, j, vreg4(wset + 4 * i), vreg4(xset + 4 * j), i, j))
-                if m < len(pending):
-                    e.read(*pending[m])
-                if m >= 8:
-                    if kk == 0 and writes:
-                        e.write(*writes[m - 8])
-                    if kk == 1 and loads:
-                        e.emit(loads[m - 8])
-                m += 1
-    if writes:
-        e.need_writes()
-    if barrier:
-        e.emit("s_barrier")
-
-
-def main_staged():
-    e = Emitter()
-    e.emit("; ======== setup ========")
-    e.emit("v_mov_b32 v%d, %%[wb]" % (ADDR + 0))
-    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (ADDR + 1))
-    e.emit("v_mov_b32 v%d, %%[xb]" % (ADDR + 2))
-    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (ADDR + 3))
-    for r in range(4):
-        e.emit("v_add_u32 v%d, 0x10000, v%d" % (ADDR + 4 + r, ADDR + r))
-    e.emit("v_mov_b32 v%d, %%[ldsw]" % LDSW)
-    e.emit("v_add_u32 v%d, 0x10000, v%d" % (LDSW + 1, LDSW))
-    e.emit("v_mov_b32 v%d, %%[wv0]" % W_VOFF)
-    e.emit("v_mov_b32 v%d, %%[xv0]" % X_VOFF)
-    for i in range(1, 4):
-        e.emit("v_add_u32 v%d, %%[w64], v%d" % (W_VOFF + i, W_VOFF + i - 1))
-        e.emit("v_add_u32 v%d, %%[x64], v%d" % (X_VOFF + i, X_VOFF + i - 1))
-    for r in range(4):
-        e.emit("v_mov_b32 v%d, 0" % (WA + r))
-    e.emit("s_nop 7")      # VALU result -> MFMA source operand needs wait states the assembler does not add
-    for i in range(4):
-        for j in range(4):
-            e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, 0" % (i, j, vreg4(WA), vreg4(WA)))
-    e.emit("; ======== prologue: tiles 0, 1 -> LDS stages 0, 1; tiles 2, 3 in flight ========")
-    e.emit("s_mov_b32 s96, 0")
-    e.emit("s_mov_b32 s98, 0")
-    for ld in load_instrs(0):
-        e.emit(ld)
-    advance_k(e)
-    for ld in load_instrs(1):
-        e.emit(ld)
-    e.emit("s_waitcnt vmcnt(0)")
-    for t in range(2):
-        for w in write_instrs(t, t):
-            e.write(*w)
-    e.need_writes()                          # the register sets are free again, the tiles are in LDS
-    advance_k(e)
-    for ld in load_instrs(0):
-        e.emit(ld)
-    advance_k(e)
-    for ld in load_instrs(1):
-        e.emit(ld)
-    e.emit("s_barrier")
-    for r in frag_reads(0, 0, WA, XA):
-        e.read(*r)
-    e.emit("s_mov_b32 s97, 4")
-    e.emit("s_cmp_ge_u32 s97, %[ht]")
-    e.emit("s_cbranch_scc1 L_tail_%=")
-    e.emit("L_loop_%=:")
-    for h in range(NSTAGE):
-        advance_k(e)
-        half_step_staged(e, h, write_vmcnt=8, do_load=True, prefetch_next=True, barrier=True)
-    e.forget_bound()
-    e.emit("s_add_u32 s97, s97, 4")
-    e.emit("s_cmp_lt_u32 s97, %[ht]")
-    e.emit("s_cbranch_scc1 L_loop_%=")
-    e.emit("L_tail_%=:")
-    e.forget_bound()
-    half_step_staged(e, 0, write_vmcnt=8, do_load=False, prefetch_next=True, barrier=True)
-    half_step_staged(e, 1, write_vmcnt=0, do_load=False, prefetch_next=True, barrier=True)
-    half_step_staged(e, 2, write_vmcnt=None, do_load=False, prefetch_next=True, barrier=False)
-    half_step_staged(e, 3, write_vmcnt=None, do_load=False, prefetch_next=False, barrier=False)
-    print("// Generated by gen_gemm_asm.py -- do not edit.")
-    for ln in e.lines:
-        print('"%s\\n"' % ln)
-
-
-
 
 
 # ---------------------------------------------------------------------------
@@ -538,7 +379,5 @@ if __name__ == "__main__":
     import sys
     if len(sys.argv) > 1 and sys.argv[1] == "half":
         main_half()
-    elif os.environ.get("CUBERT_GEMM_MODE", "dma") == "staged":
-        main_staged()
     else:
         main()
