@@ -97,7 +97,8 @@ __device__ __forceinline__ void store1(unsigned char* base, size_t elem_index, f
 // itself walks groups of kGroupM tile rows column by column: the 32 tiles that
 // an XCD's CUs hold at one time then cover 4 x 8 tiles (12 operand slabs)
 // instead of 2 x 16 (18 slabs), and the next 32 reuse the same activation rows.
-constexpr int kGroupM = 4;
+// (The 256 x 128 kernel has 64 workgroups per XCD in flight and groups 8 rows.)
+template <int kGroupM = 4>
 __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int* tn, int* tm) {
     const int xcd = pid & 7, idx = pid >> 3;
     const int base = total >> 3, rem = total & 7;
