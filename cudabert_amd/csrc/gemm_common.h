@@ -91,27 +91,42 @@ __device__ __forceinline__ void store1(unsigned char* base, size_t elem_index, f
     }
 }
 
-// Workgroup id -> (tile_n, tile_m).  Hardware hands consecutive workgroup ids
-// to the eight XCDs round-robin; the remap gives every XCD one contiguous run
-// of the tile sequence so tiles sharing operand rows share an L2.  The sequence
-// itself walks groups of kGroupM tile rows column by column: the 32 tiles that
-// an XCD's CUs hold at one time then cover 4 x 8 tiles (12 operand slabs)
-// instead of 2 x 16 (18 slabs), and the next 32 reuse the same activation rows.
-// (The 256 x 128 kernel has 64 workgroups per XCD in flight and groups 8 rows.)
+// Workgroup id -> (tile_n, tile_m).  Hardware hands consecutive workgroup ids to
+// the eight XCDs round-robin, and every XCD has its own 4 MiB L2.  When the tile
+// grid divides evenly, the XCDs own the cells of a 2 x 4 or 4 x 2 partition of it
+// (rows x columns): a quarter or half of the weight rows then stays resident in
+// an XCD's L2 and every activation row is fetched by 4 or 2 XCDs instead of all
+// operands by all.  Otherwise each XCD gets one contiguous run of the tile
+// sequence.  Inside its share an XCD walks groups of kGroupM tile rows column by
+// column, so that the tiles in flight at one time span few operand slabs and the
+// next ones reuse the same activation rows.  (kGroupM: 4 for the 256 x 256 tile
+// with 32 workgroups per XCD in flight, 8 for the 256 x 128 tile with 64.)
 template <int kGroupM = 4>
 __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int* tn, int* tm) {
     const int xcd = pid & 7, idx = pid >> 3;
-    const int base = total >> 3, rem = total & 7;
-    const int start = xcd * base + (xcd < rem ? xcd : rem);
-    const int t = start + idx;
     const int tiles_m = total / tiles_n;
-    const int per_group = kGroupM * tiles_n;
+    int xn_parts = 0;
+    if ((total & 7) == 0) {
+        if ((tiles_n & 3) == 0 && (tiles_m & 1) == 0) xn_parts = 4;
+        else if ((tiles_n & 1) == 0 && (tiles_m & 3) == 0) xn_parts = 2;
+    }
+    int n_first = 0, m_first = 0, n_count = tiles_n, m_count = tiles_m, t = idx;
+    if (xn_parts) {
+        n_count = tiles_n / xn_parts;
+        m_count = tiles_m / (8 / xn_parts);
+        n_first = (xcd % xn_parts) * n_count;
+        m_first = (xcd / xn_parts) * m_count;
+    } else {
+        const int base = total >> 3, rem = total & 7;
+        t = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    }
+    const int per_group = kGroupM * n_count;
     const int group = t / per_group, r = t - group * per_group;
-    const int left = tiles_m - group * kGroupM;
+    const int left = m_count - group * kGroupM;
     const int gm = left < kGroupM ? left : kGroupM;       // the last group may be shorter
     const int c = r / gm;
-    *tn = c;
-    *tm = group * kGroupM + (r - c * gm);
+    *tn = n_first + c;
+    *tm = m_first + group * kGroupM + (r - c * gm);
 }
 
 // The bias values a lane needs (4 NB quads) are fetched by gemm_load_bias before the
