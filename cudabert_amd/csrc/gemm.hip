@@ -11,7 +11,7 @@
 //
 // LDS image of an operand tile: two sub-blocks (the two 64-byte halves of the
 // K slab), each BT rows x 64 bytes; a row is four 16-byte chunks and chunk c
-// of row r sits in slot c ^ (((r >> 1) ^ (r >> 3)) & 3), which spreads the
+// of row r sits in slot c ^ ((r >> 2) & 3) (packed_swizzle), which spreads the
 // 16-byte fragment reads of 8 or 16 consecutive rows over all banks.  This is
 // also the on-device "packed" operand layout (common.h): a packed operand is
 // stored as 16 KiB blocks of 256 rows x 64 bytes that already are this image,
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
         const_cast<unsigned char*>(p.X), 0,
         p.x_packed ? (int)packed_bytes(p.M, p.K * ES) : (int)((((size_t)p.M - 1) * p.ldx + p.K) * ES), 0x00020000);
     const int w_rowb = p.K * ES, x_rowb = p.ldx * ES;
-    const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
+    const int dc = (lane & 3) ^ packed_swizzle(lane >> 2);     // row groups start at multiples of 16: only the lane matters
     const int w_base = p.w_packed ? ((n0 >> 8) * KB * 16384 + (n0 & 255) * 64 + wave * 1024 + lane * 16)
                                   : ((n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4));
     const int x_base = p.x_packed ? ((m0 >> 8) * KB * 16384 + (m0 & 255) * 64 + wave * 1024 + lane * 16)
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     // base + 32 i + l32 in sub-block kk >> 1.  swz(row) only depends on l32 (the
     // quadrant base and 32 i do not reach the bits it uses), so the byte offset is
     //   (off0 ^ ((kk & 1) << 5)) + (kk >> 1) * SUB + i * 2048.
-    const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
+    const int sw = packed_swizzle(l32);
     const int woff0 = (wn * (BT / 2) + l32) * 64 + ((g ^ sw) << 4);
     const int xoff0 = TILE_BYTES + (wm * (BT / 2) + l32) * 64 + ((g ^ sw) << 4);
 

@@ -52,10 +52,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     // global->LDS: one load moves 16 rows x 64 bytes.  Wave w moves the row groups w, w+4,
     // w+8, w+12 of each tile.
     //   unpacked source: lane fetches row 16*group + lane/4 and the chunk that belongs into
-    //     its LDS slot lane%4 (slot = chunk ^ swz(row)); for these groups swz only depends on
-    //     the lane and the parity of w.  One half-step further along K is +64 bytes.
+    //     its LDS slot lane%4 (slot = chunk ^ swz(row)); row groups start at multiples of 16, so
+    //     swz only depends on the lane.  One half-step further along K is +64 bytes.
     //   packed source: a tile's half-step is one contiguous 16 KiB block, the next one follows it.
-    const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
+    const int dc = (lane & 3) ^ packed_swizzle(lane >> 2);
     const int w_v0 = p.w_packed ? (tile_n * KB * 16384 + wave * 1024 + lane * 16)
                                 : ((n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4));
     const int x_v0 = p.x_packed ? (tile_m * KB * 16384 + wave * 1024 + lane * 16)
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     const int wkstep = p.w_packed ? 16384 : 64, xkstep = p.x_packed ? 16384 : 64;
     // fragment reads: chunk g of my row in the W / X tile of stage 0, k-phase 0
     const int lds_base = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
+    const int sw = packed_swizzle(l32);
     const int wb = lds_base + (wn * 128 + l32) * 64 + ((g ^ sw) << 4);
     const int xb = lds_base + 16384 + (wm * 128 + l32) * 64 + ((g ^ sw) << 4);
     const int m0b = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
     const int KB = p.K * 2 / 64;
     // One load moves 16 rows x 64 bytes.  Wave w moves the W row groups w, w+4, w+8, w+12 and the
     // X row groups w, w+4 of each tile (see the 256 x 256 kernel for the chunk choice `dc`).
-    const int dc = (lane & 3) ^ ((lane >> 3) & 3) ^ ((lane >> 5) & 1) ^ (2 * (wave & 1));
+    const int dc = (lane & 3) ^ packed_swizzle(lane >> 2);
     const int w_v0 = p.w_packed ? (tile_n * KB * 16384 + wave * 1024 + lane * 16)
                                 : ((n0 + 16 * wave + (lane >> 2)) * w_rowb + (dc << 4));
     const int x_v0 = p.x_packed ? ((m0 >> 8) * KB * 16384 + (m0 & 255) * 64 + wave * 1024 + lane * 16)
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
     const int w64 = p.w_packed ? 4096 : 64 * w_rowb, x64 = p.x_packed ? 4096 : 64 * x_rowb;
     const int wkstep = p.w_packed ? 16384 : 64, xkstep = p.x_packed ? 16384 : 64;
     const int lds_base = (int)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
-    const int sw = ((l32 >> 1) ^ (l32 >> 3)) & 3;
+    const int sw = packed_swizzle(l32);
     const int wb = lds_base + (wn * 128 + l32) * 64 + ((g ^ sw) << 4);
     const int xb = lds_base + (wm * 64 + l32) * 64 + ((g ^ sw) << 4);       // + 0x4000 is in the read offsets
     const int m0b = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);

@@ -35,7 +35,7 @@ Register plan (per lane):
   s92..s95    M0 base of stage 0..3 (stage base + wave * 1024)
 
 LDS swizzle: a tile row is 64 bytes = four 16-byte chunks; chunk c of row r sits
-in slot c ^ (((r >> 1) ^ (r >> 3)) & 3), which spreads the fragment reads of any
+in slot c ^ ((r >> 2) & 3), which spreads the fragment reads of any
 8 or 16 consecutive rows over all banks.  One buffer_load_dwordx4 ... lds moves
 16 rows (64 lanes x 16 B) to M0 + 16 * lane; the swizzle is applied on the
 global side (which chunk a lane fetches).

@@ -49,7 +49,7 @@ def packed_index(R, K):
     kbyte = (np.arange(K) * 2)[None, :]
     KB = K * 2 // 64
     rp = r & 255
-    sw = ((rp >> 1) ^ (rp >> 3)) & 3
+    sw = (rp >> 2) & 3
     off = ((r >> 8) * KB + (kbyte >> 6)) * 16384 + rp * 64 + ((((kbyte >> 4) & 3) ^ sw) << 4) + (kbyte & 15)
     return off // 2
 
