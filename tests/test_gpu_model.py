@@ -184,6 +184,28 @@ def test_base_cfg0_bf16(pb, base_dir):
     assert np.abs(pooled - pooled_ref).max() < TOL[BF16]
 
 
+@pytest.mark.parametrize("precision", [F32, BF16])
+def test_base_max_position_length(pb, base_dir, precision):
+    """Sequences at the position table's limit (S = 512) with the skewed lengths of benchmark
+    configuration 4: one long, the others short; also B = 1."""
+    wdir = str(base_dir / ("f32" if precision == F32 else "bf16"))
+    npy = W.load_npy_dir(wdir)
+    ids, seg, mask = synth.make_inputs(3, 512, [512, 40, 385], seed=44, prune=False)
+    seq_ref, pooled_ref = O.forward_torch(npy, W.BASE.heads, ids, seg, mask)
+    m = load(pb, W.BASE, wdir, precision, 3, 512)
+    try:
+        pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+        pooled1, seq1, _ = pb.encode(m, ids[:1], seg[:1], mask[:1], want_seq=True)
+    finally:
+        pb.unload_model(m)
+    print("s512 precision %d max-abs: seq %.3g pooled %.3g" % (precision, np.abs(seq - seq_ref).max(),
+                                                               np.abs(pooled - pooled_ref).max()))
+    assert np.abs(seq - seq_ref).max() < TOL[precision]
+    assert np.abs(pooled - pooled_ref).max() < TOL[precision]
+    assert np.abs(seq1[0] - seq_ref[0]).max() < TOL[precision]
+    assert np.abs(pooled1[0] - pooled_ref[0]).max() < TOL[precision]
+
+
 def test_bf16_weight_rounding_cost(pb, base_dir):
     """An arbitrary float32 checkpoint run in bf16 mode: the engine's own error
     stays as above, the rest is what rounding the weights to bfloat16 storage
