@@ -128,6 +128,19 @@ void Cuda_Bert(void* model, float* output, int* words, int* token_types, int bat
         die("Cuda_Bert");
 }
 
+void Cuda_Classify(void* model, float* output, int* words, int* token_types, int batchsize, int seq_length,
+                   int num_classes, int* attention_mask) {
+    if (!output) { cubert::set_error("output buffer is NULL"); die("Cuda_Classify"); }
+    Model* m = as_model(model, "Cuda_Classify");
+    if (m && num_classes != m->num_classes()) {
+        cubert::set_error("num_classes " + std::to_string(num_classes) + " does not match the classifier in the weight directory (" +
+                          std::to_string(m->num_classes()) + ")");
+        die("Cuda_Classify");
+    }
+    if (cubert_encode(model, words, token_types, attention_mask, batchsize, seq_length, nullptr, nullptr, output) != 0)
+        die("Cuda_Classify");
+}
+
 Retval Cuda_Inference(void* model, int* words, int* token_types, int batchsize, int seq_length, int* masks) {
     cubert::set_error("");
     Model* m = as_model(model, "Cuda_Inference");

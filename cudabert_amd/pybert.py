@@ -53,6 +53,11 @@ bert = lib.Cuda_Bert
 bert.argtypes = [c_void_p, _f32, _i32, _i32, c_int, c_int, _i32]
 bert.restype = None
 
+# the binding the reference left commented out (cuda_bert/pybert.py:40-42)
+classify = lib.Cuda_Classify
+classify.argtypes = [c_void_p, _f32, _i32, _i32, c_int, c_int, c_int, _i32]
+classify.restype = None
+
 lib.test.argtypes = [c_int, c_int, c_int, c_bool, c_int]
 lib.test.restype = None
 

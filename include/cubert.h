@@ -62,6 +62,15 @@ void Cuda_Bert(void* model, float* output, int* words, int* token_types, int bat
 Retval Cuda_Inference(void* model, int* words, int* token_types, int batchsize, int seq_length,
                       int* masks);
 
+/* The entry point the reference left commented out (cuda_bert/cuda_bert.cu:72-89; its binding
+ * cuda_bert/pybert.py:40-42): encoder + classifier head, batchsize*num_classes float32
+ * probabilities softmax(pooled @ classifier_kernel + bias) to the host buffer `output`
+ * (the head of apps/finetune.py:16-44, which keeps the last column).  Needs
+ * classifier_kernel.npy / classifier_bias.npy in the weight directory; num_classes must
+ * match them.  Synchronous; terminates the process on an invalid call like Cuda_Bert. */
+void Cuda_Classify(void* model, float* output, int* words, int* token_types, int batchsize,
+                   int seq_length, int num_classes, int* attention_mask);
+
 /* Replaces test (cuda_bert/cuda_bert.cu:91-180; cuda_bert.cuh:4-5): loads the
  * default weight directory, tiles the reference's 11-token seed input to
  * (batchsize, seq_length), runs 10 warm-up and nIter timed iterations of

@@ -99,6 +99,9 @@ def test_reference_entry_points(pb, tiny_dir):
         out = np.ones((3, W.TINY.hidden), np.float32)
         pb.bert(m, out, ids, seg, 3, 20, mask)
         assert np.abs(out - pooled_ref).max() < TOL[F32]
+        probs = np.zeros((3, 2), np.float32)
+        pb.classify(m, probs, ids, seg, 3, 20, 2, mask)           # the reference's commented-out Cuda_Classify
+        assert np.abs(probs - O.classifier_head(npy, pooled_ref)).max() < TOL[F32]
         ret = pb.inference(m, ids, seg, 3, 20, mask)
         assert ret.tensor == pb.lib.cubert_seq_ptr(m) and ret.Pooled_Output == pb.lib.cubert_pooled_ptr(m)
         pb.check(pb.lib.cubert_sync(m))
