@@ -179,3 +179,56 @@ def encode(model, ids, seg, mask=None, want_seq=False, want_cls=False):
     ptr = lambda a: None if a is None else a.ctypes.data
     check(lib.cubert_encode(model, ptr(ids), ptr(seg), ptr(mask), B, S, ptr(pooled), ptr(seq), ptr(cls)))
     return pooled, seq, cls
+
+
+# ---- the reference module's small helpers (cuda_bert/pybert.py:44-66) ----
+def filling_inputs(words, seq_length):
+    """Cycles the body of a token list (all but the last element) until the list is
+    seq_length long, keeping the last element at the end."""
+    words = list(words)
+    length = len(words) - 1
+    total = length - 1
+    end_word = words[-1]
+    words = words[:-1]
+    while total < seq_length - 2:
+        total += 1
+        words.append(words[total % length])
+    words.append(end_word)
+    return words
+
+
+def batch_inputs(row, batchsize):
+    return [row for _ in range(batchsize)]
+
+
+def warp_inputs(indexed_tokens, segments_ids, attention_masks):
+    return (numpy.array(indexed_tokens).astype(numpy.int32), numpy.array(segments_ids).astype(numpy.int32),
+            numpy.array(attention_masks).astype(numpy.int32))
+
+
+# ids of ['who', 'was', 'jim', 'henson', '?', 'jim', '[MASK]', 'was', 'a', 'puppet', '##eer'] in the
+# bert-base-uncased vocabulary: the seed input of the reference's benchmarks
+# (cuda_bert/pybert.py:75-77, cuda_bert/cuda_bert.cu:94-98)
+SEED_IDS = [2040, 2001, 3958, 27227, 1029, 3958, 103, 2001, 1037, 13997, 11510]
+SEED_SEGMENTS = [0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1]
+SEED_MASK = [1, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0]
+
+
+def test(is_large, model_dir, batchsize, seq_length, num_gpu=0, iters=100):
+    """The reference's Python timing loop (cuda_bert/pybert.py:70-100) on the seed input,
+    without its tokenizer download: prints the mean time of an asynchronous inference call."""
+    import time
+    ids, seg, mask = warp_inputs(batch_inputs(filling_inputs(SEED_IDS, seq_length), batchsize),
+                                 batch_inputs(filling_inputs(SEED_SEGMENTS, seq_length), batchsize),
+                                 batch_inputs(filling_inputs(SEED_MASK, seq_length), batchsize))
+    model = load_model(is_large, model_dir, num_gpu=num_gpu)
+    try:
+        start = time.time()
+        for _ in range(iters):
+            inference(model, ids, seg, batchsize, seq_length, mask)
+        check(lib.cubert_sync(model))
+        end = time.time()
+    finally:
+        unload_model(model)
+    print("Batchsize: {} Seq_length: {} Use_Time: {}".format(batchsize, seq_length, (end - start) / iters))
+    return (end - start) / iters

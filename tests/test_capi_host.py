@@ -152,3 +152,12 @@ def test_cuda_bert_exits_on_error_like_the_reference():
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
     assert r.returncode == 1 and "survived" not in r.stdout
     assert "Cuda_Bert failed" in r.stderr
+
+
+def test_reference_helpers(pb):
+    # cuda_bert/pybert.py:44-60
+    w = pb.filling_inputs([1, 2, 3, 9], 8)
+    assert w == [1, 2, 3, 1, 2, 3, 1, 9]
+    assert pb.filling_inputs(pb.SEED_MASK, 11) == pb.SEED_MASK
+    ids, seg, mask = pb.warp_inputs(pb.batch_inputs(w, 2), pb.batch_inputs(w, 2), pb.batch_inputs(w, 2))
+    assert ids.shape == (2, 8) and ids.dtype == np.int32
