@@ -169,6 +169,7 @@ def main():
                          "bandwidth-bound kernels (residual+LayerNorm, scale+mask+softmax, embedding+LayerNorm)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seqs", type=int, default=128, help="sequences in the CPU baseline sample")
+    ap.add_argument("--graph", action="store_true", help="replay the whole pass from a hipGraph (as small batches do by default)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the dominant kernel's launches plus one device copy of known size "
                          "(the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters); for profiler runs")
@@ -217,7 +218,7 @@ def main():
         t_gen = time.time() - t0
         t0 = time.time()
         model = pybert.load_model_ex(wdir, H, L, A, I, precision=prec, max_batchsize=B, max_seq_length=S,
-                                     graph_max_tokens=8192 if args.config == 3 else 0)
+                                     graph_max_tokens=8192 if args.config == 3 else (1 << 30 if args.graph else 0))
         t_load = time.time() - t0
     lib = pybert.lib
     if args.config == 3:

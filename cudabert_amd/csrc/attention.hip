@@ -213,32 +213,56 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const unsigned char* vb = vt + bh * 64 * (size_t)Sp * 2;
 
     // ---- stage K (rows S..Sp-1 zero), V^T and the mask row ----
-    for (int c = tid; c < Sp * 8; c += nthr) {
-        const int row = c >> 3, ch = c & 7;
-        uint4 d = {0u, 0u, 0u, 0u};
-        if (row < S) d = *reinterpret_cast<const uint4*>(kb + (size_t)c * 16);
-        *reinterpret_cast<uint4*>(sK + row * 128 + ((ch ^ (row & 7)) << 4)) = d;
-    }
+    // The workgroup has 2 Sp threads, K is 8 Sp and V^T 8 Sp 16-byte chunks: four of each per
+    // thread.  All eight loads are issued before the first LDS write so that their latencies
+    // overlap instead of adding up.
     const int vchunks = Sp >> 3;               // 16-byte chunks per V^T row
-    for (int c = tid; c < 64 * vchunks; c += nthr) {
-        const int row = c / vchunks, ch = c - row * vchunks;
-        const uint4 d = *reinterpret_cast<const uint4*>(vb + ((size_t)row * Sp + ch * 8) * 2);
-        uint2* dst = reinterpret_cast<uint2*>(sV + (size_t)row * vstride + ch * 16);     // rows are 8-byte aligned
-        dst[0] = make_uint2(d.x, d.y);
-        dst[1] = make_uint2(d.z, d.w);
+    uint4 kd[4], vd[4];
+    int vrow_i[4], vch_i[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + i * nthr;
+        kd[i] = make_uint4(0u, 0u, 0u, 0u);
+        if ((c >> 3) < S) kd[i] = *reinterpret_cast<const uint4*>(kb + (size_t)c * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + i * nthr;
+        vrow_i[i] = c / vchunks;
+        vch_i[i] = c - vrow_i[i] * vchunks;
+        vd[i] = *reinterpret_cast<const uint4*>(vb + ((size_t)vrow_i[i] * Sp + vch_i[i] * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + i * nthr;
+        const int row = c >> 3, ch = c & 7;
+        *reinterpret_cast<uint4*>(sK + row * 128 + ((ch ^ (row & 7)) << 4)) = kd[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint2* dst = reinterpret_cast<uint2*>(sV + (size_t)vrow_i[i] * vstride + vch_i[i] * 16);     // rows are 8-byte aligned
+        dst[0] = make_uint2(vd[i].x, vd[i].y);
+        dst[1] = make_uint2(vd[i].z, vd[i].w);
     }
     {
         // wave w looks at mask block w
         const float m = lane < 32 ? maskadd[(size_t)b * Sp + wave * 32 + lane] : -INFINITY;
         if (lane < 32) sM[wave * 32 + lane] = m * 1.4426950408889634f;
         const unsigned long long vis = __ballot(m > -5000.0f);
-        if (lane == 0) sLive[wave] = vis != 0ull ? 1 : 0;
+        const unsigned long long zero = __ballot(lane < 32 && m == 0.0f);
+        // bit 0: some key of the block is visible; bit 1: all 32 are, with a zero mask term
+        if (lane == 0) sLive[wave] = (vis != 0ull ? 1 : 0) | (zero == 0xffffffffull ? 2 : 0);
     }
     __syncthreads();
-    unsigned live = 0;
-    for (int i = 0; i < nblk; ++i) live |= sLive[i] ? (1u << i) : 0u;
+    unsigned live = 0, plain = 0;
+    for (int i = 0; i < nblk; ++i) {
+        const int f = sLive[i];
+        live |= (f & 1) ? (1u << i) : 0u;
+        plain |= (f & 2) ? (1u << i) : 0u;
+    }
     if (live == 0) live = 0xffffffffu;
     live = __builtin_amdgcn_readfirstlane(live);
+    plain = __builtin_amdgcn_readfirstlane(plain);
 
     // Q fragments ("B" operand: column = query), kept for the whole key loop.
     const int q0 = wave * 32;
@@ -275,34 +299,60 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
             sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf),
                                                          __builtin_bit_cast(bf16x8_t, qf[kk]), sc, 0, 0, 0);
         }
+        // Softmax with a lazily moved reference exponent: p = exp2(t - ref), where ref is the row
+        // maximum seen when it was last moved.  It only moves (and the sums are rescaled) when a
+        // block exceeds it by more than 2^20, so that in almost every block there is no rescaling
+        // of the 32 context accumulators and no second exponential; p stays below 2^20 and the
+        // final division by the row sum removes the common factor.  The first processed block
+        // (ref = -inf) always takes the move.
+        const bool is_plain = (plain >> kblk) & 1u;           // every key visible, mask term zero
         float blk_max = -INFINITY;
+        if (is_plain) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const f32x4_t m4 = *reinterpret_cast<const f32x4_t*>(sM + k0 + 8 * j + 4 * g);
+            for (int v = 0; v < 16; ++v) blk_max = fmaxf(blk_max, sc[v]);
+            blk_max *= scale_log2e;                          // scale_log2e > 0
+        } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float t = fmaf(sc[4 * j + e], scale_log2e, m4[e]);
-                sc[4 * j + e] = t;
-                blk_max = fmaxf(blk_max, t);
+            for (int j = 0; j < 4; ++j) {
+                const f32x4_t m4 = *reinterpret_cast<const f32x4_t*>(sM + k0 + 8 * j + 4 * g);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = fmaf(sc[4 * j + e], scale_log2e, m4[e]);
+                    sc[4 * j + e] = t;
+                    blk_max = fmaxf(blk_max, t);
+                }
             }
         }
         blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
-        const float new_max = fmaxf(run_max, blk_max);    // finite: a processed block holds a real key column
-        const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);
-        float blk_sum = 0.0f;
+        if (__ballot(blk_max > run_max + 20.0f) != 0ull) {    // finite blk_max: a processed block holds a real key column
+            const float new_max = fmaxf(run_max, blk_max);
+            const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);     // 1 for the lanes that stay
+            run_sum *= alpha;
+            run_max = new_max;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const float pv = __builtin_amdgcn_exp2f(sc[v] - new_max);
-            sc[v] = pv;
-            blk_sum += pv;
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+        }
+        float blk_sum = 0.0f;
+        if (is_plain) {
+            const float neg_ref = -run_max;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float pv = __builtin_amdgcn_exp2f(fmaf(sc[v], scale_log2e, neg_ref));
+                sc[v] = pv;
+                blk_sum += pv;
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float pv = __builtin_amdgcn_exp2f(sc[v] - run_max);
+                sc[v] = pv;
+                blk_sum += pv;
+            }
         }
         blk_sum += __shfl_xor(blk_sum, 32);
-        run_sum = run_sum * alpha + blk_sum;
-        run_max = new_max;
-#pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+        run_sum += blk_sum;
 
         // ---- ctx^T += V^T (rows = head features) x P^T (column = my query) ----
 #pragma unroll
@@ -350,6 +400,7 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
     const int cp = ctx_packed ? 1 : 0;
     if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
     if (B <= 0 || heads <= 0 || S <= 0) { set_error("attention: empty problem"); return false; }
+    if (!(scale > 0.0f)) { set_error("attention: scale must be positive"); return false; }
     if (Sp % 32 != 0 || Sp < S || Sp - S >= 32) {
         set_error("attention: Sp must be S rounded up to a multiple of 32");
         return false;
