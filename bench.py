@@ -54,10 +54,10 @@ def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
     def ffn_in():
         pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H, prec,
                                         out_elt, 1, 0, gflags, st.cuda_stream))
-    for _ in range(3):
+    for _ in range(20):          # enough launches for the clocks to settle
         ffn_in()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    launches = 20
+    launches = 50
     e0.record(st)
     for _ in range(launches):
         ffn_in()
