@@ -432,3 +432,68 @@ def test_pooler(pb, w_elt):
                                      stream()))
     torch.cuda.synchronize()
     assert np.abs(out.cpu().numpy() - ref).max() < 2e-5, np.abs(out.cpu().numpy() - ref).max()
+
+
+def test_gemm_random_shapes(pb):
+    """Seeded sweep over irregular shapes: every tile choice (0 = the library's own), both operand
+    types, row-major operands, edge tiles in both dimensions."""
+    rng = np.random.default_rng(2024)
+    for case in range(36):
+        elt = BF16 if case % 3 else F32
+        M = int(rng.integers(1, 700))
+        N = int(rng.integers(1, 130)) * 8
+        K = int(rng.integers(1, 12)) * 64
+        epi = int(rng.integers(0, 3))
+        tile = [0, 64, 128, 256, 384][case % 5]
+        if tile == 384 and elt == F32:
+            tile = 0
+        print("gemm sweep", case, elt, M, N, K, epi, tile, flush=True)
+        X = rng.standard_normal((M, K)).astype(np.float32)
+        Wt = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+        b = rng.standard_normal(N).astype(np.float32)
+        tdt = torch.float32 if elt == F32 else torch.bfloat16
+        if elt == BF16:
+            X, Wt = bf16_round(X), bf16_round(Wt)
+        ref = X.astype(np.float64) @ Wt.astype(np.float64).T + b
+        ref = gelu64(ref) if epi == 1 else (np.tanh(ref) if epi == 2 else ref)
+        Xd, Wd, bd = dev(X, tdt), dev(Wt, tdt), dev(b)
+        # guard rows around Y: nothing outside [M, N] may be written
+        Y = torch.full((M + 2, N), 7.0, device="cuda")
+        pb.check(pb.lib.cubert_op_gemm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Y[1:].data_ptr(), M, N, K, K, elt, F32,
+                                       epi, tile, 0, stream()))
+        torch.cuda.synchronize()
+        got = Y.cpu().numpy().astype(np.float64)
+        assert (got[0] == 7.0).all() and (got[-1] == 7.0).all(), case
+        assert np.abs(got[1:-1] - ref).max() < 3e-4 * max(1.0, np.sqrt(K / 256)), (case, np.abs(got[1:-1] - ref).max())
+
+
+def test_attention_random_shapes(pb):
+    """Seeded sweep over batch, length, head count and arbitrary (non-prefix) masks, bf16."""
+    rng = np.random.default_rng(77)
+    for case in range(12):
+        B, S, heads = int(rng.integers(1, 5)), int(rng.integers(1, 300)), int(rng.integers(1, 5))
+        Sp = (S + 31) // 32 * 32
+        print("attention sweep", case, B, S, heads, flush=True)
+        q = bf16_round(rng.standard_normal((B, heads, S, 64)).astype(np.float32))
+        k = bf16_round(rng.standard_normal((B, heads, S, 64)).astype(np.float32))
+        v = bf16_round(rng.standard_normal((B, heads, S, 64)).astype(np.float32))
+        mask = (rng.random((B, S)) < rng.random((B, 1))).astype(np.float32)
+        mask[:, int(rng.integers(0, S))] = 1
+        sc = np.einsum("bhsd,bhtd->bhst", q.astype(np.float64), k.astype(np.float64)) * 0.125
+        sc = sc + ((1.0 - mask) * -10000.0)[:, None, None, :]
+        sc = sc - sc.max(-1, keepdims=True)
+        p = np.exp(sc)
+        p /= p.sum(-1, keepdims=True)
+        ref = np.einsum("bhst,bhtd->bshd", p, v.astype(np.float64)).reshape(B * S, heads * 64)
+        vt = np.zeros((B, heads, 64, Sp), np.float32)
+        vt[..., :S] = v.transpose(0, 1, 3, 2)
+        maskadd = np.full((B, Sp), -np.inf, np.float32)
+        maskadd[:, :S] = (1.0 - mask) * -10000.0
+        qd, kd, vd, md = dev(q, torch.bfloat16), dev(k, torch.bfloat16), dev(vt, torch.bfloat16), dev(maskadd)
+        ctx = torch.full((B * S, heads * 64), float("nan"), dtype=torch.bfloat16, device="cuda")
+        pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), ctx.data_ptr(),
+                                            B, heads, S, 0.125, BF16, 0, stream()))
+        torch.cuda.synchronize()
+        got = ctx.float().cpu().numpy()
+        assert np.isfinite(got).all(), case
+        assert np.abs(got - ref).max() < 2e-2, (case, np.abs(got - ref).max())
