@@ -159,8 +159,8 @@ def extras_leg(torch, pybert, model, ids, seg, mask, dims, prec, steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--precision", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4],
                     help="2 = headline; 3 = latency regime (B=1 and 8, hipGraph replay, p50/p99)")
