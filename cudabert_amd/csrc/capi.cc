@@ -56,6 +56,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
     opt.varlen = env_int("CUBERT_VARLEN", 0) != 0;
     opt.split_k = env_int("CUBERT_SPLIT_K", 1) != 0;
+    opt.fuse_residual = env_int("CUBERT_FUSE_RESIDUAL", 1) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;
@@ -281,6 +282,17 @@ int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 
+int cubert_op_gemm_residual(const void* X, const void* W, const float* bias, const float* R, float* Y, int M, int N,
+                            int K, int ldx, int elt, int tile, int flags, void* stream) {
+    cubert::set_error("");
+    if (!R) { cubert::set_error("cubert_op_gemm_residual: null residual"); return 1; }
+    cubert::GemmParams p;
+    p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.elt = elt;
+    p.out_elt = cubert::kF32; p.epilogue = cubert::kEpiBias; p.tile = tile; p.residual = R;
+    apply_gemm_flags(&p, flags);
+    return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
 int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q, void* k, void* vt, int B, int S,
                        int heads, int elt, int tile, int flags, void* stream) {
     cubert::set_error("");
@@ -310,7 +322,8 @@ int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gam
     return cubert::launch_add_layernorm(x, y, y_elt, gamma, beta, static_cast<cubert::bf16_t*>(xb),
                                         (flags & CUBERT_Y_PACKED) != 0, rows, hidden,
                                         static_cast<hipStream_t>(stream),
-                                        CUBERT_SPLITS_OF(flags) > 1 ? CUBERT_SPLITS_OF(flags) : 1) ? 0 : 1;
+                                        CUBERT_SPLITS_OF(flags) > 1 ? CUBERT_SPLITS_OF(flags) : 1,
+                                        (flags & CUBERT_LN_NO_RESIDUAL) == 0) ? 0 : 1;
 }
 
 int cubert_op_embed_layernorm(const int* ids, const int* seg, const int* mask, const float* word, const float* pos,

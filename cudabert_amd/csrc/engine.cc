@@ -459,6 +459,8 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         return sp;
     };
     const int sp_ao = splits_for(H), sp_fo = splits_for(I);
+    // the attn-out / FFN-out GEMMs add the residual stream in their epilogue, so LayerNorm reads one operand
+    const bool fuse_res = opt_.fuse_residual;
 
     if (!mark(kPhEmbed)) return false;
     const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
@@ -481,9 +483,10 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;
         g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_ao;
+        g.residual = fuse_res ? x32 : nullptr;
         if (!mark(kPhAttnOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st, sp_ao)) return false;
+        if (!launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st, sp_ao, !fuse_res)) return false;
         // feed-forward
         g = GemmParams();
         g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h;
@@ -492,9 +495,10 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = h; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32;
         g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_fo;
+        g.residual = fuse_res ? x32 : nullptr;
         if (!mark(kPhFFNOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st, sp_fo)) return false;
+        if (!launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st, sp_fo, !fuse_res)) return false;
     }
     // pooler: first-token gather + dense + tanh on the float32 sequence output
     if (!mark(kPhPooler)) return false;

@@ -26,6 +26,7 @@ struct ModelOptions {
     int max_seq = 0;
     int split_parts = 2;           // number of parts (1..4) a large batch is cut into
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
+    bool fuse_residual = true;     // residual add in the epilogue of the GEMM before each LayerNorm
     bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
     bool varlen = false;           // host-input calls with prefix masks compute only the valid tokens
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)

@@ -229,10 +229,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #undef CUBERT_K_STEP
 
     f32x4_t bias[4 * NB];      // fetched here rather than before the loop: no registers to spare there
-    constexpr bool SPLITK = EPI == kEpiBias && OUT == kF32;      // the only combination launch_gemm splits
-    gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
+    constexpr bool SPLITK = (EPI == kEpiBias || EPI == kEpiBiasRes) && OUT == kF32;      // the only combinations launch_gemm splits
+    if constexpr (!gemm_bias_at_readout<OUT, EPI>()) gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
     // every wave is past the last step's barrier: the tiles are dead, lds0 is free for staging
-    gemm_epilogue<OUT, EPI, NB, NB, SPLITK>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
+    gemm_epilogue<OUT, EPI, NB, NB, SPLITK, 4, true>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
 }
 
 template <int ELT, int OUT, int EPI, int BT, int NS = 2>
@@ -264,6 +264,9 @@ bool launch_epi(const GemmDev& d, int epi, int bt, hipStream_t stream) {
         case kEpiBiasTanh: return launch_tile<ELT, OUT, kEpiBiasTanh>(d, bt, stream);
         case kEpiQKV: return launch_tile<ELT, OUT, kEpiQKV>(d, bt, stream);
         case kEpiQKVMap: return launch_tile<ELT, OUT, kEpiQKVMap>(d, bt, stream);
+        case kEpiBiasRes:
+            if constexpr (OUT == kF32) return launch_tile<ELT, OUT, kEpiBiasRes>(d, bt, stream);
+            break;
     }
     set_error("gemm: unknown epilogue");
     return false;
@@ -331,8 +334,17 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     d.M = p.M; d.N = p.N; d.K = p.K; d.ldx = p.ldx;
     d.x_packed = p.x_packed; d.w_packed = p.w_packed; d.y_packed = p.y_packed;
     int out = p.out_elt;
-    const int epi = (p.epilogue == kEpiQKV && p.rowmap) ? (int)kEpiQKVMap : p.epilogue;
-    if (p.epilogue == kEpiQKVMap) { set_error("gemm: unknown epilogue"); return false; }
+    int epi = (p.epilogue == kEpiQKV && p.rowmap) ? (int)kEpiQKVMap : p.epilogue;
+    if (p.epilogue == kEpiQKVMap || p.epilogue == kEpiBiasRes) { set_error("gemm: unknown epilogue"); return false; }
+    if (p.residual) {
+        if (p.epilogue != kEpiBias || out != kF32 || p.y_packed || p.N % 4 != 0 ||
+            (reinterpret_cast<uintptr_t>(p.residual) & 15)) {
+            set_error("gemm: a residual needs the plain bias epilogue, a float32 row-major result, N a multiple of 4 and 16-byte alignment");
+            return false;
+        }
+        epi = kEpiBiasRes;
+        d.R = p.residual;
+    }
     if (p.epilogue == kEpiQKV) {
         if (!p.q || !p.k || !p.vt || p.S <= 0 || p.heads <= 0 || p.N != 3 * p.heads * 64 ||
             (!p.rowmap && p.M % p.S != 0) || p.Sp < p.S || p.Sp % 4 != 0) {
@@ -356,7 +368,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     }
     d.splits = p.splits > 0 ? p.splits : 1;
     if (d.splits > 1) {
-        if (epi != kEpiBias || out != kF32 || p.y_packed || d.splits > p.K / bk) {
+        if ((epi != kEpiBias && epi != kEpiBiasRes) || out != kF32 || p.y_packed || d.splits > p.K / bk) {
             set_error("gemm: split K needs the plain bias epilogue, a float32 result and at least one K step per split");
             return false;
         }

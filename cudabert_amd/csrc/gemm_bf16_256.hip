@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
 
     f32x16_t acc[4][4];       // zeroed inside the asm block
     f32x4_t bias[16];
-    gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
+    if constexpr (!gemm_bias_at_readout<OUT, EPI>()) gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
 
     asm volatile(
 #include "gemm_bf16_256_loop.inc"
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
 
     // Stages 0 and 1 were last read two barriers ago; the tail of the loop only reads stages
     // 2 and 3, so the first 64 KiB are free for the epilogue's staging while slower waves finish.
-    gemm_epilogue<OUT, EPI, 4, 4>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
+    gemm_epilogue<OUT, EPI, 4, 4, false, 8, true>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
 }
 
 // ---------------------------------------------------------------------------
@@ -154,8 +154,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
 
     // The block ends with all loads landed and a barrier: the whole LDS is free for staging.
     f32x4_t bias[16];
-    gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
-    gemm_epilogue<OUT, EPI, 4, 2>(p, acc, bias, n0 + wn * 128, m0 + wm * 64, l32, g, lds + wave * 16384);
+    if constexpr (!gemm_bias_at_readout<OUT, EPI>()) gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
+    gemm_epilogue<OUT, EPI, 4, 2, false, 8, true>(p, acc, bias, n0 + wn * 128, m0 + wm * 64, l32, g, lds + wave * 16384);
 }
 
 template <int OUT>
@@ -167,6 +167,12 @@ bool launch_epi_half(const GemmDev& d, int epi, hipStream_t stream) {
         case kEpiBiasTanh: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBiasTanh>), grid, block, 0, stream, d); break;
         case kEpiQKV: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiQKV>), grid, block, 0, stream, d); break;
         case kEpiQKVMap: hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiQKVMap>), grid, block, 0, stream, d); break;
+        case kEpiBiasRes:
+            if constexpr (OUT == kF32) {
+                hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBiasRes>), grid, block, 0, stream, d);
+                break;
+            }
+            [[fallthrough]];
         default: set_error("gemm: unknown epilogue"); return false;
     }
     CUBERT_HIP_OK(hipGetLastError());
@@ -182,6 +188,12 @@ bool launch_epi(const GemmDev& d, int epi, hipStream_t stream) {
         case kEpiBiasTanh: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasTanh>), grid, block, 0, stream, d); break;
         case kEpiQKV: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiQKV>), grid, block, 0, stream, d); break;
         case kEpiQKVMap: hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiQKVMap>), grid, block, 0, stream, d); break;
+        case kEpiBiasRes:
+            if constexpr (OUT == kF32) {
+                hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasRes>), grid, block, 0, stream, d);
+                break;
+            }
+            [[fallthrough]];
         default: set_error("gemm: unknown epilogue"); return false;
     }
     CUBERT_HIP_OK(hipGetLastError());

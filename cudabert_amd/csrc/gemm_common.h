@@ -25,6 +25,7 @@ struct GemmDev {
     int tiles_n, tiles_m;
     int x_packed, w_packed, y_packed;     // operand / result in the packed layout (common.h)
     const int* rowmap;                    // QKV epilogue: row m -> token b * S + s (nullptr: m itself)
+    const float* R;                       // kEpiBiasRes: [M, N] float32 row-major, added to the result
     int splits;                           // split K: blockIdx.y owns a K range, results go to Y + y * M * N (f32)
 };
 
@@ -129,6 +130,12 @@ __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, i
     *tm = m_first + group * kGroupM + (r - c * gm);
 }
 
+// float32 results without an activation take their bias in the read-out phase of the epilogue, where
+// a lane serves one group of four features for all rows (one quad instead of 4 NB): gemm_load_bias is
+// not needed for them and the epilogue ignores its `bias` argument.
+template <int OUT, int EPI>
+constexpr bool gemm_bias_at_readout() { return OUT == kF32 && (EPI == kEpiBias || EPI == kEpiBiasRes); }
+
 // The bias values a lane needs (4 NB quads) are fetched by gemm_load_bias before the
 // K loop so that their latency is hidden; features past N read the last valid quad
 // (their results are never stored).
@@ -146,7 +153,12 @@ __device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int
 // SPLITK: the launch may have several workgroups per tile (blockIdx.y = K share), each writing
 // its partial result to its own copy of Y.
 // The wave's quadrant is NBI x NBJ accumulator blocks (features x tokens).
-template <int OUT, int EPI, int NBI, int NBJ, bool SPLITK = false>
+//
+// kEpiBiasRes (float32 row-major result): the read-out adds R[m][n] to every element, fetched in the
+// layout of the stores (whole row segments).  The fetches go out RPB read-out steps at a time; with RDB
+// the next batch is requested before the current one is consumed (two batches of registers), which a
+// kernel with one workgroup per CU needs because nothing else covers the latency there.
+template <int OUT, int EPI, int NBI, int NBJ, bool SPLITK = false, int RPB = 4, bool RDB = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NBI][NBJ], const f32x4_t (&bias)[4 * NBI],
                                               int n_base, int m_base, int l32, int g, unsigned char* scratch) {
     constexpr int OES = (OUT == kBF16) ? 2 : 4;
@@ -154,8 +166,35 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
     constexpr int CH = RB / 16;             // 16-byte chunks per row
     constexpr int RPI = 64 / CH;            // rows one store instruction covers
     constexpr int EPC = 16 / OES;           // elements per chunk
+    constexpr bool RES = EPI == kEpiBiasRes;
+    static_assert(!RES || OUT == kF32, "the residual epilogue writes float32");
+    constexpr int NIT = 32 / RPI;                               // read-out steps per block column
+    constexpr int PB = RES ? (NIT < RPB ? NIT : RPB) : NIT;     // steps per residual batch
+    constexpr int NBATCH = NIT / PB;
     const int lane = l32 + 32 * g;
     const int rrow = lane / CH, rc = lane % CH;
+    f32x4_t res[RES && RDB ? 2 : 1][PB];
+    bool addres = RES;
+    if constexpr (SPLITK) addres = RES && blockIdx.y == 0;      // split K: the residual is added once
+    // rows / features outside the matrix fetch a valid neighbour; their sums are never stored
+    auto fetch_res = [&](int j, int bt, f32x4_t (&r)[PB]) {
+#pragma unroll
+        for (int s = 0; s < PB; ++s) {
+            const int mm = m_base + 32 * j + (bt * PB + s) * RPI + rrow;
+            const int n = n_base + rc * EPC;
+            r[s] = *reinterpret_cast<const f32x4_t*>(p.R + (size_t)(mm < p.M ? mm : p.M - 1) * p.N + (n < p.N ? n : p.N - 4));
+        }
+    };
+    if constexpr (RES && RDB)
+        if (addres) fetch_res(0, 0, res[0]);
+    constexpr bool BIAS_RO = gemm_bias_at_readout<OUT, EPI>();
+    f32x4_t bias_ro = {0.0f, 0.0f, 0.0f, 0.0f};
+    if constexpr (BIAS_RO) {
+        bool addb = true;
+        if constexpr (SPLITK) addb = blockIdx.y == 0;           // split K: the bias is added once
+        const int n = n_base + rc * EPC;
+        if (addb) bias_ro = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
+    }
     // compact rows: the token of this lane's row in every block row, fetched together up front;
     // the read-out phase takes a row's token from the lane that owns it
     int tokj[NBJ];
@@ -183,11 +222,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             for (int qd = 0; qd < 4; ++qd) {
                 const int fq = 32 * i + 8 * qd + 4 * g;          // feature within the quadrant
                 const int n = n_base + fq;
-                const f32x4_t b4 = bias[4 * i + qd];
+                f32x4_t b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                if constexpr (!BIAS_RO) b4 = bias[4 * i + qd];
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float t = acc[i][j][4 * qd + e] + b4[e];
+                    float t = acc[i][j][4 * qd + e];
+                    if constexpr (!BIAS_RO) t += b4[e];
                     if constexpr (EPI == kEpiBiasGelu) t = (OUT == kBF16) ? gelu_fast(t) : gelu_erf(t);
                     if constexpr (EPI == kEpiBiasTanh) t = tanhf(t);
                     v[e] = t;
@@ -209,9 +250,23 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             }
         }
 #pragma unroll
-        for (int s = 0; s < 32 / RPI; ++s) {
+        for (int s = 0; s < NIT; ++s) {
             const int row = s * RPI + rrow;
-            const u32x4_t d = *reinterpret_cast<const u32x4_t*>(buf + row * RB + (((rc ^ row) & (CH - 1)) << 4));
+            u32x4_t d = *reinterpret_cast<const u32x4_t*>(buf + row * RB + (((rc ^ row) & (CH - 1)) << 4));
+            if constexpr (RES) {
+                const int batch = j * NBATCH + s / PB;          // compile-time after unrolling
+                if (s % PB == 0 && addres) {
+                    if constexpr (RDB) {
+                        if (batch + 1 < NBJ * NBATCH) fetch_res((batch + 1) / NBATCH, (batch + 1) % NBATCH, res[(batch + 1) & 1]);
+                    } else {
+                        fetch_res(j, s / PB, res[0]);
+                    }
+                }
+                if (addres) d = __builtin_bit_cast(u32x4_t, (__builtin_bit_cast(f32x4_t, d) + bias_ro) + res[RDB ? (batch & 1) : 0][s % PB]);
+                else d = __builtin_bit_cast(u32x4_t, __builtin_bit_cast(f32x4_t, d) + bias_ro);
+            } else if constexpr (BIAS_RO) {
+                d = __builtin_bit_cast(u32x4_t, __builtin_bit_cast(f32x4_t, d) + bias_ro);
+            }
             const int mm = m_base + 32 * j + row;
             const int n = n_base + rc * EPC;
             int tok = mm;

@@ -23,6 +23,7 @@ enum GemmEpilogue : int {
     kEpiBiasTanh = 2,  // Y = tanh(acc + bias)           (ops/elementwise.cu:56-61 fused)
     kEpiQKV = 3,       // scatter into per-head Q, K and transposed V (see below)
     kEpiQKVMap = 4,    // the same on compact rows: row m is token rowmap[m] (chosen by launch_gemm when rowmap is set)
+    kEpiBiasRes = 5,   // Y = acc + bias + R, float32 row-major (chosen by launch_gemm when residual is set)
 };
 
 // Unpadded ("compact") rows: only the valid tokens of every sequence are stored,
@@ -54,6 +55,9 @@ struct GemmParams {
     void* vt = nullptr;
     int S = 0, Sp = 0, heads = 0;
     const int* rowmap = nullptr;   // kEpiQKV on compact rows: row m is token rowmap[m] = b * S + s
+    // kEpiBias with a float32 row-major Y: [M, N] float32 added to the result (the residual branch of
+    // the layer, so that the LayerNorm after it reads one operand).  With split K it goes into partial 0.
+    const float* residual = nullptr;
     int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile) or kTile256x128
     // Split K (kEpiBias, float32 Y): `splits` workgroups share a tile, each reduces its share of K and
     // writes its partial result to Y + z * M * N; the bias goes into partial 0.  The consumer adds
@@ -85,9 +89,11 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
 // LayerNorm).  eps = 1e-12 inside the square root, biased variance
 // (cuda_bert/ops/layernorm.cu:136-182; modeling.py:168-172).
 // xb_packed: write the copy in the packed GEMM-operand layout (common.h).
+// add_x = false: x <- LayerNorm(y): y is already the sum with the residual stream (a GEMM with
+// GemmParams::residual produced it) and x is only written.
 bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
                           const float* beta, bf16_t* xb, bool xb_packed, int rows, int H,
-                          hipStream_t stream, int y_parts = 1);
+                          hipStream_t stream, int y_parts = 1, bool add_x = true);
 
 // --------------------------------------------------- embedding + LN --------
 // x[t] = LayerNorm(word[ids[t]] + pos[t % S] + type[seg[t]]); also writes the

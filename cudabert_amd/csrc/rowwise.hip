@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
                                                             const float* __restrict__ gamma,
                                                             const float* __restrict__ beta,
                                                             bf16_t* __restrict__ xb, int rows, int H,
-                                                            int xb_packed, int y_parts) {
+                                                            int xb_packed, int y_parts, int add_x) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -84,7 +84,10 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
     for (int c = 0; c < kMaxChunks; ++c) {
         const int i = c * 256 + lane * 4;
         if (i < H) {
-            f32x4_t a = *reinterpret_cast<const f32x4_t*>(xrow + i);
+            // add_x == 0: y already holds the sum with the residual stream (the producing GEMM added it),
+            // x is only written
+            f32x4_t a = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (YELT == -1 || add_x) a = *reinterpret_cast<const f32x4_t*>(xrow + i);
             if constexpr (YELT == kF32) {
                 // the addend may come as several partial sums (split-K GEMM), [part][rows][H]
                 f32x4_t t = *reinterpret_cast<const f32x4_t*>(y + ((size_t)row * H + i) * 4);
@@ -445,7 +448,8 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 }  // namespace
 
 bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta,
-                          bf16_t* xb, bool xb_packed, int rows, int H, hipStream_t stream, int y_parts) {
+                          bf16_t* xb, bool xb_packed, int rows, int H, hipStream_t stream, int y_parts, bool add_x) {
+    if (!add_x && !y) { set_error("layernorm: without the residual stream an addend is required"); return false; }
     if (y_parts < 1 || (y_parts > 1 && (!y || y_elt != kF32))) { set_error("layernorm: partial addends must be float32"); return false; }
     if (xb && xb_packed && H % 32 != 0) { set_error("layernorm: a packed copy needs H to be a multiple of 32"); return false; }
     const int xp = xb_packed ? 1 : 0;
@@ -460,9 +464,9 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
     }
     dim3 grid((rows + 3) / 4), block(256);
     const unsigned char* yc = static_cast<const unsigned char*>(y);
-    if (!y) hipLaunchKernelGGL(add_layernorm_kernel<-1>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts);
-    else if (y_elt == kF32) hipLaunchKernelGGL(add_layernorm_kernel<kF32>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts);
-    else if (y_elt == kBF16) hipLaunchKernelGGL(add_layernorm_kernel<kBF16>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts);
+    if (!y) hipLaunchKernelGGL(add_layernorm_kernel<-1>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
+    else if (y_elt == kF32) hipLaunchKernelGGL(add_layernorm_kernel<kF32>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
+    else if (y_elt == kBF16) hipLaunchKernelGGL(add_layernorm_kernel<kBF16>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
     else { set_error("layernorm: bad addend type"); return false; }
     CUBERT_HIP_OK(hipGetLastError());
     return true;

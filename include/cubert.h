@@ -162,6 +162,7 @@ long cubert_capacity_tokens(void* model);
 #define CUBERT_W_PACKED 2           /* weight operand W is packed */
 #define CUBERT_Y_PACKED 4           /* write Y packed (bf16 output only) */
 #define CUBERT_COMPILER_SCHEDULED 8 /* 256 tile: general kernel instead of the hand-scheduled one */
+#define CUBERT_LN_NO_RESIDUAL 16    /* cubert_op_add_layernorm: y already contains the residual stream */
 /* Split K (cubert_op_gemm, epilogue 0, float32 Y): n workgroups share a tile, each reduces 1/n of K
  * and writes its partial sum to Y + i * M * N (the bias is in partial 0); Y holds n * M * N floats and
  * the consumer adds the parts (cubert_op_add_layernorm takes the count in the same flag bits). */
@@ -176,6 +177,12 @@ size_t cubert_packed_offset(int row, int byte_in_row, int row_bytes);
  * op_Tanh (ops/elementwise.cu:37-70). */
 int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int M, int N, int K,
                    int ldx, int elt, int out_elt, int epilogue, int tile, int flags, void* stream);
+
+/* Y[M,N] (float32) = X * W^T + bias + R[M,N] (float32): the linear before a LayerNorm with the
+ * residual add of cuApplyLayerNorm (cuda_bert/ops/layernorm.cu:152-158) moved into its epilogue.
+ * With CUBERT_SPLITS(n) the residual and the bias are in partial 0. */
+int cubert_op_gemm_residual(const void* X, const void* W, const float* bias, const float* R, float* Y,
+                            int M, int N, int K, int ldx, int elt, int tile, int flags, void* stream);
 
 /* Fused QKV projection (op_BatchedLinear::forward, cuda_bert/ops/linear.cu:241-319):
  * X[B*S, hidden] * Wqkv[3*hidden, hidden]^T + bias -> q,k [B,heads,S,64],
@@ -193,7 +200,8 @@ int cubert_op_attention(const void* q, const void* k, const void* vt, const floa
  * cuda_bert/ops/layernorm.cu:136-206). */
 int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma,
                             const float* beta, void* xb, int rows, int hidden, int flags,
-                            void* stream); /* flags: CUBERT_Y_PACKED writes xb packed */
+                            void* stream); /* flags: CUBERT_Y_PACKED writes xb packed;
+                                              CUBERT_LN_NO_RESIDUAL: x <- LayerNorm(y), x is only written */
 
 /* Embedding gather + add + LayerNorm + additive mask rows (Embedding::forward,
  * cuda_bert/ops/embedding.cu:3-58). */
