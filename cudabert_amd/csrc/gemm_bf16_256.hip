@@ -68,7 +68,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     const int wb = lds_base + (wn * 128 + l32) * 64 + ((g ^ sw) << 4);
     const int xb = lds_base + 16384 + (wm * 128 + l32) * 64 + ((g ^ sw) << 4);
     const int m0b = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
-    const int ldsw = lds_base + wave * 1024 + lane * 16;      // where my 16 bytes of a loaded row group go
     const int ht = p.K / 32;          // half-steps; a multiple of 4
 
     f32x16_t acc[4][4];       // zeroed inside the asm block
@@ -79,12 +78,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
 #include "gemm_bf16_256_loop.inc"
         : CUBERT_ACC_OPERANDS
         : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
-          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep),
-          [ldsw] "v"(ldsw)
-        : "memory", "scc", "s92", "s93", "s94", "s95", "s96", "s97", "s98", CUBERT_V10(10), CUBERT_V10(11), CUBERT_V10(12), CUBERT_V10(13), CUBERT_V10(14), CUBERT_V10(15),
-          "v160", "v161", "v162", "v163", "v170", "v171", "v176", "v177", "v178", "v179",
-          CUBERT_V10(18), CUBERT_V10(19), CUBERT_V10(20), CUBERT_V10(21), CUBERT_V10(22), CUBERT_V10(23),
-          CUBERT_V10(24), "v250", "v251", "v252", "v253", "v254", "v255");
+          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep)
+        : "memory", "scc", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "v96", "v97", "v98", "v99",
+          CUBERT_V10(10), CUBERT_V10(11), CUBERT_V10(12), CUBERT_V10(13), CUBERT_V10(14), CUBERT_V10(15), CUBERT_V10(16),
+          "v170", "v171", "v172", "v173", "v174", "v175");
 
     // Stages 0 and 1 were last read two barriers ago; the tail of the loop only reads stages
     // 2 and 3, so the first 64 KiB are free for the epilogue's staging while slower waves finish.

@@ -26,11 +26,13 @@ what lets half-step h prefetch tile h+1's fragments before its own barrier.
 
 Register plan (per lane):
   a[0:255]    accumulators: 4x4 blocks of 32x32 (inline-asm "+a" operands)
-  v[192:207]  W fragments, set A (block i at 192+4i)   v[208:223]  X fragments, set A
-  v[224:239]  W fragments, set B                       v[240:255]  X fragments, set B
-  v[176:179]  LDS byte addresses of my fragment row in stage 0: W k-phase 0, W k-phase 1,
-              X k-phase 0, X k-phase 1                 v[180:183]  the same + 65536 (stages 2, 3)
-  v[184:187]  global lane offsets of my 4 W row groups v[188:191]  same for X
+  v[112:127]  W fragments, set A (block i at 112+4i)   v[128:143]  X fragments, set A
+  v[144:159]  W fragments, set B                       v[160:175]  X fragments, set B
+  v[96:99]    LDS byte addresses of my fragment row in stage 0: W k-phase 0, W k-phase 1,
+              X k-phase 0, X k-phase 1                 v[100:103]  the same + 65536 (stages 2, 3)
+  v[104:107]  global lane offsets of my 4 W row groups v[108:111]  same for X
+  (the registers above v175 stay free: with 256 accumulators the wave then leaves room on its
+  SIMD for waves of small kernels from another stream)
   s96 / s98 K byte offset of the W / X tile being fetched, s97 loop counter,
   s92..s95    M0 base of stage 0..3 (stage base + wave * 1024)
 
@@ -40,9 +42,9 @@ in slot c ^ ((r >> 2) & 3), which spreads the fragment reads of any
 16 rows (64 lanes x 16 B) to M0 + 16 * lane; the swizzle is applied on the
 global side (which chunk a lane fetches).
 """
-WA, XA, WB, XB = 192, 208, 224, 240
-ADDR = 176            # + 4 * bank + {0: W kk0, 1: W kk1, 2: X kk0, 3: X kk1}
-W_VOFF, X_VOFF = 184, 188
+WA, XA, WB, XB = 112, 128, 144, 160
+ADDR = 96             # + 4 * bank + {0: W kk0, 1: W kk1, 2: X kk0, 3: X kk1}
+W_VOFF, X_VOFF = 104, 108
 NSTAGE = 4
 
 
