@@ -249,6 +249,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 store4<OUT>(buf + l32 * RB + ((((fb >> 4) ^ l32) & (CH - 1)) << 4) + (fb & 15), 0, v);
             }
         }
+        // Results leave with non-temporal stores: they are not read again by this kernel, and kept out of
+        // the way they evict less of the operand slabs the XCD's other tiles are still reading (the
+        // FFN-in launch fetches 20 % less through L2 with them).
 #pragma unroll
         for (int s = 0; s < NIT; ++s) {
             const int row = s * RPI + rrow;
@@ -278,13 +281,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 const int which = n >= p.hidden ? 1 : 0;
                 const int hn = n - which * p.hidden;
                 const size_t bh = (size_t)b2 * p.heads + (hn >> 6);
-                *reinterpret_cast<u32x4_t*>((which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES) = d;
+                __builtin_nontemporal_store(d, reinterpret_cast<u32x4_t*>((which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES));
             } else if (p.y_packed) {
                 // packed bf16 result: the next GEMM's activation operand
-                *reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)) = d;
+                __builtin_nontemporal_store(d, reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)));
             } else {
                 const size_t part = SPLITK ? (size_t)blockIdx.y * p.M : 0;
-                *reinterpret_cast<u32x4_t*>(p.Y + ((part + mm) * p.N + n) * OES) = d;
+                __builtin_nontemporal_store(d, reinterpret_cast<u32x4_t*>(p.Y + ((part + mm) * p.N + n) * OES));
             }
         }
     }
