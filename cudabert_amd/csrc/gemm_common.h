@@ -251,7 +251,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
         }
         // Results leave with non-temporal stores: they are not read again by this kernel, and kept out of
         // the way they evict less of the operand slabs the XCD's other tiles are still reading (the
-        // FFN-in launch fetches 20 % less through L2 with them).
+        // FFN-in launch fetches 20 % less through L2 with them).  q and k keep ordinary stores: the
+        // attention kernel that follows reads them at once and measured faster with them cached.
 #pragma unroll
         for (int s = 0; s < NIT; ++s) {
             const int row = s * RPI + rrow;
@@ -281,7 +282,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 const int which = n >= p.hidden ? 1 : 0;
                 const int hn = n - which * p.hidden;
                 const size_t bh = (size_t)b2 * p.heads + (hn >> 6);
-                __builtin_nontemporal_store(d, reinterpret_cast<u32x4_t*>((which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES));
+                *reinterpret_cast<u32x4_t*>((which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES) = d;
             } else if (p.y_packed) {
                 // packed bf16 result: the next GEMM's activation operand
                 __builtin_nontemporal_store(d, reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)));
