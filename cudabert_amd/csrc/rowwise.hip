@@ -57,7 +57,7 @@ __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H
             f32x4_t o;
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[e] = g4[e] * (v[c][e] * rstd) + b4[e];
-            *reinterpret_cast<f32x4_t*>(xrow + i) = o;
+            __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t*>(xrow + i));
             if (xb) {
                 bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
                 unsigned char* dst = reinterpret_cast<unsigned char*>(xb);
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
             if (YELT == -1 || add_x) a = *reinterpret_cast<const f32x4_t*>(xrow + i);
             if constexpr (YELT == kF32) {
                 // the addend may come as several partial sums (split-K GEMM), [part][rows][H]
-                f32x4_t t = *reinterpret_cast<const f32x4_t*>(y + ((size_t)row * H + i) * 4);
+                f32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(y + ((size_t)row * H + i) * 4));
                 for (int part = 1; part < y_parts; ++part)
                     t += *reinterpret_cast<const f32x4_t*>(y + (((size_t)part * rows + row) * H + i) * 4);
                 a += t;
