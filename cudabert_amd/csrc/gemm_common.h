@@ -182,7 +182,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
         for (int s = 0; s < PB; ++s) {
             const int mm = m_base + 32 * j + (bt * PB + s) * RPI + rrow;
             const int n = n_base + rc * EPC;
-            r[s] = *reinterpret_cast<const f32x4_t*>(p.R + (size_t)(mm < p.M ? mm : p.M - 1) * p.N + (n < p.N ? n : p.N - 4));
+            r[s] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p.R + (size_t)(mm < p.M ? mm : p.M - 1) * p.N + (n < p.N ? n : p.N - 4)));
         }
     };
     if constexpr (RES && RDB)
