@@ -358,6 +358,10 @@ def test_large_headline_shape(pb, tmp_path):
         assert np.abs(pooled[:n] - pooled_ref).max() < TOL[BF16]
         assert np.abs(cls[:n] - O.classifier_head(npy, pooled_ref)).max() < TOL[BF16]
         assert np.isfinite(seq).all() and np.allclose(cls.sum(1), 1.0, atol=1e-5)
+        # the two half-batches run on two streams: repeated calls must not differ in a single bit
+        for _ in range(5):
+            pooled_r, seq_r, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+            assert np.array_equal(pooled_r, pooled) and np.array_equal(seq_r, seq)
         perm = np.random.default_rng(1).permutation(B)
         pooled_p, seq_p, _ = pb.encode(m, ids[perm], seg[perm], mask[perm], want_seq=True)
         assert np.array_equal(pooled_p, pooled[perm]) and np.array_equal(seq_p, seq[perm])
