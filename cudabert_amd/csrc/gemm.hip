@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     const int l32 = lane & 31, g = lane >> 5;
 
     int tile_n, tile_m;
-    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, &tile_n, &tile_m);
+    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
     const int n0 = tile_n * BT, m0 = tile_m * BT;
 
     // ---- global -> LDS, asynchronous, no registers in between ----
@@ -379,10 +379,12 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         if (p.elt != kBF16 || d.splits != 1) { set_error("gemm: the 256x128 tile is bf16 only and does not split K"); return false; }
         d.tiles_n = (p.N + 255) / 256;
         d.tiles_m = (p.M + 127) / 128;
+        d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 8);
         return launch_gemm_bf16_t256x128(d, out, epi, stream);
     }
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
+    d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 4);
     if (p.elt == kBF16) {
         // 256 tile with a multiple of four half-steps: the hand-scheduled kernel
         if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled && d.splits == 1)

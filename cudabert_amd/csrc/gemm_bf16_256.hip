@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     const int l32 = lane & 31, g = lane >> 5;
 
     int tile_n, tile_m;
-    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, &tile_n, &tile_m);
+    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
     const int n0 = tile_n * BT, m0 = tile_m * BT;
 
     // Buffer descriptors as plain SGPR quads: base, base_hi (stride 0), num_records, flags.
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
     const int l32 = lane & 31, g = lane >> 5;
 
     int tile_n, tile_m;
-    tile_of_block<8>(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, &tile_n, &tile_m);
+    tile_of_block<8>(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
     const int n0 = tile_n * 256, m0 = tile_m * 128;
 
     const unsigned long long wa = reinterpret_cast<unsigned long long>(p.W);

@@ -24,6 +24,7 @@ struct GemmDev {
     int S, Sp, heads, hidden;
     int tiles_n, tiles_m;
     int x_packed, w_packed, y_packed;     // operand / result in the packed layout (common.h)
+    int xn_parts;                         // how the XCDs divide the tile grid (tile_of_block)
     const int* rowmap;                    // QKV epilogue: row m -> token b * S + s (nullptr: m itself)
     const float* R;                       // kEpiBiasRes: [M, N] float32 row-major, added to the result
     int splits;                           // split K: blockIdx.y owns a K range, results go to Y + y * M * N (f32)
@@ -93,24 +94,22 @@ __device__ __forceinline__ void store1(unsigned char* base, size_t elem_index, f
 }
 
 // Workgroup id -> (tile_n, tile_m).  Hardware hands consecutive workgroup ids to
-// the eight XCDs round-robin, and every XCD has its own 4 MiB L2.  When the tile
-// grid divides evenly, the XCDs own the cells of a 2 x 4 or 4 x 2 partition of it
-// (rows x columns): a quarter or half of the weight rows then stays resident in
-// an XCD's L2 and every activation row is fetched by 4 or 2 XCDs instead of all
-// operands by all.  Otherwise each XCD gets one contiguous run of the tile
-// sequence.  Inside its share an XCD walks groups of kGroupM tile rows column by
+// the eight XCDs round-robin, and every XCD has its own 4 MiB L2.  xn_parts = 4 or
+// 2 (chosen by gemm_pick_partition on the host, only when the grid divides): the
+// XCDs own the cells of a 2 x 4 or 4 x 2 partition of the tile grid (rows x
+// columns), so a quarter or half of the weight rows stays resident in an XCD's L2
+// and every activation row is fetched by 4 or 2 XCDs.  xn_parts = 0: each XCD gets
+// one contiguous run of the tile sequence, i.e. a band of token rows with all the
+// weight columns: activations are fetched once, the weights stream through every
+// XCD.  Inside its share an XCD walks groups of kGroupM tile rows column by
 // column, so that the tiles in flight at one time span few operand slabs and the
 // next ones reuse the same activation rows.  (kGroupM: 4 for the 256 x 256 tile
 // with 32 workgroups per XCD in flight, 8 for the 256 x 128 tile with 64.)
 template <int kGroupM = 4>
-__device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int* tn, int* tm) {
+__device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, int xn_parts, int* tn, int* tm) {
     const int xcd = pid & 7, idx = pid >> 3;
     const int tiles_m = total / tiles_n;
-    int xn_parts = 0;
-    if ((total & 7) == 0) {
-        if ((tiles_n & 3) == 0 && (tiles_m & 1) == 0) xn_parts = 4;
-        else if ((tiles_n & 1) == 0 && (tiles_m & 3) == 0) xn_parts = 2;
-    }
+    if (xn_parts && ((total & 7) != 0 || tiles_n % xn_parts != 0 || tiles_m % (8 / xn_parts) != 0)) xn_parts = 0;
     int n_first = 0, m_first = 0, n_count = tiles_n, m_count = tiles_m, t = idx;
     if (xn_parts) {
         n_count = tiles_n / xn_parts;
@@ -128,6 +127,28 @@ __device__ __forceinline__ void tile_of_block(int pid, int total, int tiles_n, i
     const int c = r / gm;
     *tn = n_first + c;
     *tm = m_first + group * kGroupM + (r - c * gm);
+}
+
+// Host side of tile_of_block: the partition with the smaller estimated traffic between memory and
+// the L2s.  A 2-D partition fetches the activations xn_parts times and each XCD's share of the
+// weights once if it fits beside the streaming activations (else once per group of tile rows); a
+// contiguous run fetches the activations once and streams all the weights through every XCD once
+// per group.  x_bytes / w_bytes: size of the operands; group_m: the kernel's kGroupM.
+inline int gemm_pick_partition(double x_bytes, double w_bytes, int tiles_n, int tiles_m, int group_m) {
+    const double l2_fit = 2.5 * 1024 * 1024;
+    auto groups = [&](int rows) { return (double)((rows + group_m - 1) / group_m); };
+    const int rows_per_xcd = (tiles_m + 7) / 8;
+    double best = x_bytes + 8.0 * w_bytes * (w_bytes <= l2_fit ? 1.0 : groups(rows_per_xcd));
+    int pick = 0;
+    if ((((long)tiles_n * tiles_m) & 7) == 0) {
+        for (int xn = 2; xn <= 4; xn += 2) {
+            if (tiles_n % xn != 0 || tiles_m % (8 / xn) != 0) continue;
+            const double share = w_bytes / xn;
+            const double f = x_bytes * xn + share * 8.0 * (share <= l2_fit ? 1.0 : groups(tiles_m / (8 / xn)));
+            if (f < best) { best = f; pick = xn; }
+        }
+    }
+    return pick;
 }
 
 // float32 results without an activation take their bias in the read-out phase of the epilogue, where
