@@ -3,6 +3,7 @@
 // load-time weight transpose.  One wave64 owns one row; reductions are
 // butterfly shuffles over the 64 lanes, no LDS.
 #include "kernels.h"
+#include <type_traits>
 
 namespace cubert {
 namespace {
@@ -89,9 +90,8 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
             f32x4_t a = {0.0f, 0.0f, 0.0f, 0.0f};
             if (YELT == -1 || add_x) a = *reinterpret_cast<const f32x4_t*>(xrow + i);
             if constexpr (YELT == kF32) {
-                // the addend may come as several partial sums (split-K GEMM), [part][rows][H]
                 f32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(y + ((size_t)row * H + i) * 4));
-                for (int part = 1; part < y_parts; ++part)
+                for (int part = 1; part < y_parts; ++part)     // partial sums of a split-K GEMM, [part][rows][H]
                     t += *reinterpret_cast<const f32x4_t*>(y + (((size_t)part * rows + row) * H + i) * 4);
                 a += t;
             } else if constexpr (YELT == kBF16) {
@@ -99,6 +99,53 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) a[e] += (float)t[e];
             }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[c][e] = a[e];
+        }
+    }
+    normalise_store(v, H, lane, gamma, beta, xrow, xb, row, xb_packed);
+}
+
+// The same operation for a short batch whose addend comes as the partial sums of a split-K GEMM
+// ([part][rows][H] float32): one workgroup per row, so that the few rows still spread over the
+// chip and every partial sum is requested in one round trip.  Wave w adds up the parts of features
+// 256 w .. 256 w + 255; wave 0 then normalises the row with exactly the arithmetic of
+// add_layernorm_kernel (same per-lane values, same reduction order).
+__global__ __launch_bounds__(256) void add_layernorm_parts_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                  const float* __restrict__ gamma,
+                                                                  const float* __restrict__ beta,
+                                                                  bf16_t* __restrict__ xb, int rows, int H,
+                                                                  int xb_packed, int y_parts, int add_x) {
+    __shared__ f32x4_t sums[kMaxChunks][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = blockIdx.x;
+    float* xrow = x + (size_t)row * H;
+    const int i = wave * 256 + lane * 4;
+    if (i < H) {
+        f32x4_t a = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (add_x) a = *reinterpret_cast<const f32x4_t*>(xrow + i);
+        f32x4_t t = *reinterpret_cast<const f32x4_t*>(y + (size_t)row * H + i);
+        for (int p0 = 1; p0 < y_parts; p0 += 8) {
+            f32x4_t u[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int part = p0 + j < y_parts ? p0 + j : 0;        // a repeat of part 0 is not added
+                u[j] = *reinterpret_cast<const f32x4_t*>(y + ((size_t)part * rows + row) * H + i);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (p0 + j < y_parts) t += u[j];
+        }
+        a += t;
+        sums[wave][lane] = a;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float v[kMaxChunks][4];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+        if (c * 256 + lane * 4 < H) {
+            const f32x4_t a = sums[c][lane];
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[c][e] = a[e];
         }
@@ -383,8 +430,8 @@ __global__ void fill_f32_kernel(float* dst, float value, size_t n) {
 
 // pooled[b, n] = tanh(bias[n] + sum_k x[b * S, k] * W[n, k]): the first-token
 // gather (row stride S*H of the float32 sequence output), the dense layer and
-// the tanh in one pass.  A workgroup handles one batch row and 64 outputs; each
-// wave 16 outputs, lanes split K.  W is [H, H] row-major ([out, in]).
+// the tanh in one pass.  A workgroup handles one batch row and 16 outputs; each
+// wave 4 outputs, lanes split K.  W is [H, H] row-major ([out, in]).
 template <int ELT>
 __global__ __launch_bounds__(256) void pooler_kernel(const float* __restrict__ x, const unsigned char* __restrict__ W,
                                                      const float* __restrict__ bias, float* __restrict__ pooled,
@@ -402,27 +449,34 @@ __global__ __launch_bounds__(256) void pooler_kernel(const float* __restrict__ x
             for (int e = 0; e < 4; ++e) xv[c][e] = t[e];
         }
     }
-    for (int o = 0; o < 16; ++o) {
-        const int n = blockIdx.y * 64 + wave * 16 + o;
-        if (n >= H) break;
+    // the wave's four weight rows are requested together: a one-sequence batch has nothing else to
+    // hide the latency behind
+    constexpr int WES = ELT == kBF16 ? 2 : 4;
+    typedef typename std::conditional<ELT == kBF16, bf16x4_t, f32x4_t>::type wvec_t;
+    wvec_t w4[4][kMaxChunks];
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+        const int n = blockIdx.y * 16 + wave * 4 + o;
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c) {
+            const int i = c * 256 + lane * 4;
+            if (i < H) w4[o][c] = *reinterpret_cast<const wvec_t*>(W + ((size_t)(n < H ? n : H - 1) * H + i) * WES);
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+        const int n = blockIdx.y * 16 + wave * 4 + o;
         float acc = 0.0f;
 #pragma unroll
         for (int c = 0; c < kMaxChunks; ++c) {
             const int i = c * 256 + lane * 4;
             if (i < H) {
-                if constexpr (ELT == kBF16) {
-                    const bf16x4_t w4 = *reinterpret_cast<const bf16x4_t*>(W + ((size_t)n * H + i) * 2);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc += xv[c][e] * (float)w4[e];
-                } else {
-                    const f32x4_t w4 = *reinterpret_cast<const f32x4_t*>(W + ((size_t)n * H + i) * 4);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc += xv[c][e] * w4[e];
-                }
+                for (int e = 0; e < 4; ++e) acc += xv[c][e] * (float)w4[o][c][e];
             }
         }
         acc = wave_sum(acc);
-        if (lane == 0) pooled[(size_t)b * H + n] = tanhf(acc + bias[n]);
+        if (lane == 0 && n < H) pooled[(size_t)b * H + n] = tanhf(acc + bias[n]);
     }
 }
 
@@ -465,6 +519,7 @@ bool launch_add_layernorm(float* x, const void* y, int y_elt, const float* gamma
     dim3 grid((rows + 3) / 4), block(256);
     const unsigned char* yc = static_cast<const unsigned char*>(y);
     if (!y) hipLaunchKernelGGL(add_layernorm_kernel<-1>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
+    else if (y_elt == kF32 && y_parts > 1) hipLaunchKernelGGL(add_layernorm_parts_kernel, dim3(rows), block, 0, stream, x, static_cast<const float*>(y), gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
     else if (y_elt == kF32) hipLaunchKernelGGL(add_layernorm_kernel<kF32>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
     else if (y_elt == kBF16) hipLaunchKernelGGL(add_layernorm_kernel<kBF16>, grid, block, 0, stream, x, yc, gamma, beta, xb, rows, H, xp, y_parts, add_x ? 1 : 0);
     else { set_error("layernorm: bad addend type"); return false; }
@@ -561,7 +616,7 @@ bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, 
     }
     if (!x || !W || !bias || !pooled || !aligned16(x) || !aligned16(W)) { set_error("pooler: null or misaligned operand"); return false; }
     if (B > 65535) { set_error("pooler: batch too large"); return false; }
-    dim3 grid(B, (H + 63) / 64), block(256);
+    dim3 grid(B, (H + 15) / 16), block(256);
     const unsigned char* wc = static_cast<const unsigned char*>(W);
     if (w_elt == kBF16) hipLaunchKernelGGL(pooler_kernel<kBF16>, grid, block, 0, stream, x, wc, bias, pooled, S, H, cu);
     else if (w_elt == kF32) hipLaunchKernelGGL(pooler_kernel<kF32>, grid, block, 0, stream, x, wc, bias, pooled, S, H, cu);
