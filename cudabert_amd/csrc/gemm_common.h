@@ -270,11 +270,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 store4<OUT>(buf + l32 * RB + ((((fb >> 4) ^ l32) & (CH - 1)) << 4) + (fb & 15), 0, v);
             }
         }
-        // float32 row-major results leave with non-temporal stores: they are read once, by a row kernel,
-        // and kept out of the way they evict less of the operand slabs the XCD's other tiles are still
-        // reading.  Results that the next kernel reads as a GEMM or attention operand (q, k, packed
-        // bf16) keep ordinary stores: the whole pass measured faster with them cached, although a
-        // launch on its own fetches 20 % less through L2 when they are non-temporal too.
+        // Results leave with ordinary stores: the next kernel reads them at once (as an operand, or the
+        // LayerNorm its addend) and the whole pass measured faster with them cached, although a launch
+        // on its own fetches 20 % less through L2 when they are non-temporal.
 #pragma unroll
         for (int s = 0; s < NIT; ++s) {
             const int row = s * RPI + rrow;
@@ -310,7 +308,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                 *reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)) = d;
             } else {
                 const size_t part = SPLITK ? (size_t)blockIdx.y * p.M : 0;
-                __builtin_nontemporal_store(d, reinterpret_cast<u32x4_t*>(p.Y + ((part + mm) * p.N + n) * OES));
+                *reinterpret_cast<u32x4_t*>(p.Y + ((part + mm) * p.N + n) * OES) = d;
             }
         }
     }
