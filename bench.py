@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --roofline-only`, each
 # counter scaled by what it reads for a 256 MiB device copy (2.0 and 1.0); the summary
 # with the commands is profiles/ffn_in_gemm_cfg2_bf16_pmc.txt.
-MEASURED_TRAFFIC = {("bf16", 25600, 4096, 1024): 6.368e8}
+MEASURED_TRAFFIC = {("bf16", 25600, 4096, 1024): 6.354e8}
 
 
 def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
