@@ -16,6 +16,8 @@
 // context comes out transposed too: a lane holds one query and four
 // consecutive head features per accumulator quad -> vector stores into the
 // row-major [tokens, hidden] context matrix.
+#include <atomic>
+
 #include "kernels.h"
 
 namespace cubert {
@@ -420,13 +422,15 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
         const int vstride = round_up(Sp * 2, 256) + 8;
         const size_t lds = (size_t)Sp * 128 + 64 * (size_t)vstride + (size_t)Sp * 4 + 64;
         // More than 64 KiB of dynamic LDS has to be allowed once per device.
-        static bool allowed[64] = {};
+        // (Several host threads, one model each, may get here together: the flag is atomic and
+        // setting the attribute twice is harmless.)
+        static std::atomic<bool> allowed[64];
         int dev = 0;
         CUBERT_HIP_OK(hipGetDevice(&dev));
-        if (dev < 0 || dev >= 64 || !allowed[dev]) {
+        if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
             CUBERT_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_lds_kernel),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            if (dev >= 0 && dev < 64) allowed[dev] = true;
+            if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
         }
         hipLaunchKernelGGL(attention_lds_kernel, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd, cc,
                            heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);

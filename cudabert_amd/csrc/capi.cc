@@ -52,6 +52,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.dims.inter = cfg.intermediate;
     opt.precision = cfg.precision;
     opt.graph_max_tokens = cfg.graph_max_tokens;
+    opt.graph_cache = env_int("CUBERT_GRAPH_CACHE", 64);
     opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
     opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
     opt.varlen = env_int("CUBERT_VARLEN", 0) != 0;
@@ -254,6 +255,7 @@ void test(int batchsize, int seq_length, int nIter, bool large, int num_gpu) {
     std::printf(" 99 Latency : %fms\n", latency[std::min(nIter - 1, (int)(nIter * 0.99))]);
     std::printf(" Throughput: %f lines per second\n", nIter * 1000.0 / total);
     std::printf("Time= %.2f(ms)\n\n", total / nIter);
+    std::fflush(stdout);
     (void)hipEventDestroy(start);
     (void)hipEventDestroy(stop);
     release_model(model);

@@ -2,6 +2,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <iterator>
 
 #include "kernels.h"
 #include "weights.h"
@@ -369,14 +370,24 @@ bool Model::run(int B, int S, bool has_mask) {
     last_compact_ = false;
     const long tokens = (long)B * S;
     if (opt_.graph_max_tokens <= 0 || tokens > opt_.graph_max_tokens) return enqueue(B, S, has_mask);
-    const long key = ((long)B * 1024 + S) * 2 + (has_mask ? 1 : 0);
-    GraphEntry& ge = graphs_[key];
-    if (ge.exec) {
-        CUBERT_HIP_OK(hipGraphLaunch(ge.exec, stream_));
+    // One entry per (B, S, mask) shape; the key is injective for every B <= 1024 and any S.
+    const unsigned long long key = ((unsigned long long)B << 33) | ((unsigned long long)(unsigned)S << 1) | (has_mask ? 1ull : 0ull);
+    auto it = graphs_.find(key);
+    if (it != graphs_.end() && it->second.exec) {
+        it->second.last_use = ++graph_clock_;
+        CUBERT_HIP_OK(hipGraphLaunch(it->second.exec, stream_));
         return true;
     }
-    if (ge.seen++ == 0) return enqueue(B, S, has_mask);      // first sight: run eagerly (one-time kernel setup)
-    // second sight: capture the launch sequence, then replay it
+    if (it == graphs_.end()) {
+        // first sight: run eagerly (one-time kernel setup) and remember the shape
+        if (graphs_.size() >= 4 * (size_t)max_graphs()) forget_uncaptured_shapes();
+        graphs_[key].last_use = ++graph_clock_;
+        return enqueue(B, S, has_mask);
+    }
+    // second sight: capture the launch sequence, then replay it.  The cache holds at most
+    // max_graphs() instantiated graphs; the least recently used one makes room.
+    if (!evict_graphs(max_graphs() - 1)) return false;
+    GraphEntry& ge = graphs_[key];
     hipGraph_t graph = nullptr;
     CUBERT_HIP_OK(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal));
     const bool ok = enqueue(B, S, has_mask);
@@ -387,8 +398,39 @@ bool Model::run(int B, int S, bool has_mask) {
     const hipError_t e2 = hipGraphInstantiate(&ge.exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     if (e2 != hipSuccess) { ge.exec = nullptr; set_error(std::string("hipGraphInstantiate failed: ") + hipGetErrorString(e2)); return false; }
+    ge.last_use = ++graph_clock_;
     CUBERT_HIP_OK(hipGraphLaunch(ge.exec, stream_));
     return true;
+}
+
+int Model::graphs_cached() const {
+    int n = 0;
+    for (const auto& kv : graphs_) n += kv.second.exec ? 1 : 0;
+    return n;
+}
+
+// Destroys least recently used graphs until at most `keep` remain.  A graph may still be
+// running on the stream, so the stream is drained first (evictions are rare).
+bool Model::evict_graphs(int keep) {
+    int have = graphs_cached();
+    if (have <= keep) return true;
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    while (have > keep) {
+        auto lru = graphs_.end();
+        for (auto it = graphs_.begin(); it != graphs_.end(); ++it)
+            if (it->second.exec && (lru == graphs_.end() || it->second.last_use < lru->second.last_use)) lru = it;
+        if (lru == graphs_.end()) break;
+        (void)hipGraphExecDestroy(lru->second.exec);
+        graphs_.erase(lru);
+        --have;
+    }
+    return true;
+}
+
+// Shapes seen once and never again would otherwise pile up in the map.
+void Model::forget_uncaptured_shapes() {
+    for (auto it = graphs_.begin(); it != graphs_.end();)
+        it = it->second.exec ? std::next(it) : graphs_.erase(it);
 }
 
 // One forward pass.  A large batch is cut into parts of whole sequences that run

@@ -30,6 +30,7 @@ struct ModelOptions {
     bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
     bool varlen = false;           // host-input calls with prefix masks compute only the valid tokens
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
+    int graph_cache = 64;          // instantiated hipGraphs kept per model (least recently used is dropped)
     std::string dir;
 };
 
@@ -75,7 +76,7 @@ class Model {
     long capacity_tokens() const { return cap_tokens_; }
     int last_batch() const { return B_; }
     int last_seq() const { return S_; }
-    int graphs_cached() const { return (int)graphs_.size(); }
+    int graphs_cached() const;                         // instantiated hipGraphs held
     size_t weight_bytes() const { return weight_bytes_; }
     size_t activation_bytes() const { return act_bytes_; }
 
@@ -125,8 +126,14 @@ class Model {
     bool last_compact_ = false;
     int cur_parts_ = 1;          // parts of the pass being enqueued
     int B_ = 0, S_ = 0;
-    struct GraphEntry { hipGraphExec_t exec = nullptr; int seen = 0; };
-    std::map<long, GraphEntry> graphs_;
+    // hipGraph cache: one entry per (B, S, mask) shape, captured on second sight, at most
+    // opt_.graph_cache instantiated at a time (least recently used goes first).
+    int max_graphs() const { return opt_.graph_cache > 0 ? opt_.graph_cache : 1; }
+    struct GraphEntry { hipGraphExec_t exec = nullptr; unsigned long long last_use = 0; };
+    std::map<unsigned long long, GraphEntry> graphs_;
+    unsigned long long graph_clock_ = 0;
+    bool evict_graphs(int keep);
+    void forget_uncaptured_shapes();
     bool profiling_ = false;
     std::vector<hipEvent_t> prof_events_;
     std::vector<int> prof_phase_;

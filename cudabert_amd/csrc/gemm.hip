@@ -113,10 +113,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
     const int kt0 = (int)((long)steps * blockIdx.y / p.splits);
     const int KT = (int)((long)steps * (blockIdx.y + 1) / p.splits);
     // A K step past the end (odd step counts run one phantom step) fetches from
-    // beyond the descriptor's range and therefore fills the tile with zeros.
+    // beyond the descriptor's range and therefore fills the tile with zeros: bit 31 of
+    // the lane offset puts it past any descriptor (launch_gemm keeps operands below 2 GiB).
 #define CUBERT_ISSUE_TILE(BUF, kt)                                                                          \
     do {                                                                                                    \
-        const int oob = (kt) < KT ? 0 : 0x40000000;                                                         \
+        const int oob = (kt) < KT ? 0 : (int)0x80000000u;                                                   \
         _Pragma("unroll") for (int i = 0; i < GROUPS; ++i) {                                                \
             const int sb = (4 * i) / SBDIV, gq = (4 * i) % SBDIV;                                       \
             __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                       \

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
         : CUBERT_ACC_OPERANDS
         : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
           [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep)
-        : "memory", "scc", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "v96", "v97", "v98", "v99",
+        : "memory", "scc", "m0", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "v96", "v97", "v98", "v99",
           CUBERT_V10(10), CUBERT_V10(11), CUBERT_V10(12), CUBERT_V10(13), CUBERT_V10(14), CUBERT_V10(15), CUBERT_V10(16),
           "v170", "v171", "v172", "v173", "v174", "v175");
 
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
         : CUBERT_ACC_OPERANDS_H
         : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
           [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep)
-        : "memory", "scc", "s92", "s93", "s94", "s96", "s97", "s98", "v64", "v65", "v66", "v67", "v68", "v69",
+        : "memory", "scc", "m0", "s92", "s93", "s94", "s96", "s97", "s98", "v64", "v65", "v66", "v67", "v68", "v69",
           CUBERT_V10(7), CUBERT_V10(8), CUBERT_V10(9), CUBERT_V10(10), CUBERT_V10(11), "v120", "v121", "v122",
           "v123", "v124", "v125");
 

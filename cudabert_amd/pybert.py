@@ -183,54 +183,43 @@ def encode(model, ids, seg, mask=None, want_seq=False, want_cls=False):
     return pooled, seq, cls
 
 
-# ---- the reference module's small helpers (cuda_bert/pybert.py:44-66) ----
-def filling_inputs(words, seq_length):
-    """Cycles the body of a token list (all but the last element) until the list is
-    seq_length long, keeping the last element at the end."""
-    words = list(words)
-    length = len(words) - 1
-    total = length - 1
-    end_word = words[-1]
-    words = words[:-1]
-    while total < seq_length - 2:
-        total += 1
-        words.append(words[total % length])
-    words.append(end_word)
-    return words
-
-
-def batch_inputs(row, batchsize):
-    return [row for _ in range(batchsize)]
-
-
-def warp_inputs(indexed_tokens, segments_ids, attention_masks):
-    return (numpy.array(indexed_tokens).astype(numpy.int32), numpy.array(segments_ids).astype(numpy.int32),
-            numpy.array(attention_masks).astype(numpy.int32))
-
-
+# ---- benchmark input of the reference (cuda_bert/pybert.py:44-100, cuda_bert/cuda_bert.cu:94-103) ----
 # ids of ['who', 'was', 'jim', 'henson', '?', 'jim', '[MASK]', 'was', 'a', 'puppet', '##eer'] in the
-# bert-base-uncased vocabulary: the seed input of the reference's benchmarks
-# (cuda_bert/pybert.py:75-77, cuda_bert/cuda_bert.cu:94-98)
+# bert-base-uncased vocabulary, their segment ids and mask.
 SEED_IDS = [2040, 2001, 3958, 27227, 1029, 3958, 103, 2001, 1037, 13997, 11510]
 SEED_SEGMENTS = [0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1]
 SEED_MASK = [1, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0]
 
 
+def seed_batch(batchsize, seq_length):
+    """The reference benchmarks' input as int32 [batchsize, seq_length] arrays (ids, segments, mask):
+    each 11-entry seed row is stretched to seq_length by cycling through its first ten entries and
+    keeping its last entry in the last column, and the row is repeated batchsize times."""
+    if seq_length < 2:
+        raise ValueError("seq_length must be at least 2")
+    cycle = numpy.arange(seq_length - 1) % 10
+
+    def stretch(seed):
+        seed = numpy.asarray(seed, numpy.int32)
+        row = numpy.append(seed[cycle], seed[-1])
+        return numpy.ascontiguousarray(numpy.broadcast_to(row, (batchsize, seq_length)))
+
+    return stretch(SEED_IDS), stretch(SEED_SEGMENTS), stretch(SEED_MASK)
+
+
 def test(is_large, model_dir, batchsize, seq_length, num_gpu=0, iters=100):
-    """The reference's Python timing loop (cuda_bert/pybert.py:70-100) on the seed input,
-    without its tokenizer download: prints the mean time of an asynchronous inference call."""
+    """Mean time of an asynchronous inference call on the seed batch: what the reference's
+    Python timing loop prints (cuda_bert/pybert.py:70-100), without its tokenizer download."""
     import time
-    ids, seg, mask = warp_inputs(batch_inputs(filling_inputs(SEED_IDS, seq_length), batchsize),
-                                 batch_inputs(filling_inputs(SEED_SEGMENTS, seq_length), batchsize),
-                                 batch_inputs(filling_inputs(SEED_MASK, seq_length), batchsize))
+    ids, seg, mask = seed_batch(batchsize, seq_length)
     model = load_model(is_large, model_dir, num_gpu=num_gpu)
     try:
-        start = time.time()
+        start = time.perf_counter()
         for _ in range(iters):
             inference(model, ids, seg, batchsize, seq_length, mask)
         check(lib.cubert_sync(model))
-        end = time.time()
+        mean = (time.perf_counter() - start) / iters
     finally:
         unload_model(model)
-    print("Batchsize: {} Seq_length: {} Use_Time: {}".format(batchsize, seq_length, (end - start) / iters))
-    return (end - start) / iters
+    print("Batchsize: {} Seq_length: {} Use_Time: {}".format(batchsize, seq_length, mean))
+    return mean

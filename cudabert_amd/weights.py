@@ -98,6 +98,20 @@ def synth_state(dims: BertDims, seed: int = 20240, degenerate: bool = True,
     return sd
 
 
+def bf16_representable(state: Dict[str, np.ndarray]) -> Dict[str, np.ndarray]:
+    """The same checkpoint with every Linear kernel (2-D, not an embedding table) rounded to the
+    nearest bfloat16 and stored as float32 again: the tensors the engine's bf16 mode keeps in
+    bfloat16.  A float32 model and the bf16 engine then hold identical weights, so that a
+    comparison between them measures the arithmetic and not the storage rounding."""
+    import torch
+    out = {}
+    for name, arr in state.items():
+        if arr.ndim == 2 and "embeddings" not in name:
+            arr = torch.from_numpy(np.ascontiguousarray(arr)).to(torch.bfloat16).to(torch.float32).numpy()
+        out[name] = arr
+    return out
+
+
 def convert_name(name: str, ndim: int) -> str:
     """PyTorch parameter name -> ``.npy`` base name
     (convert_pytorch_model_to_npys.py:27-40)."""

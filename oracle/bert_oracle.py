@@ -77,13 +77,11 @@ def extended_mask_torch(mask):
     return (1.0 - mask.to(torch.float32)).unsqueeze(1).unsqueeze(2) * -10000.0
 
 
-def self_attention_torch(x, npy, p, heads, ext_mask, rnd=None):
-    """modeling.py:222-253.  ``rnd`` optionally rounds stage outputs (used only
-    by the reduced-precision plan emulation below)."""
+def self_attention_torch(x, npy, p, heads, ext_mask):
+    """modeling.py:222-253."""
     import torch
     B, S, H = x.shape
     d = H // heads
-    r = rnd or (lambda t: t)
 
     def lin(name):
         return x @ _t(npy, p + f"attention_self_{name}_kernel") + _t(npy, p + f"attention_self_{name}_bias")
@@ -91,27 +89,25 @@ def self_attention_torch(x, npy, p, heads, ext_mask, rnd=None):
     def split(t):                     # transpose_for_scores, modeling.py:222-225
         return t.view(B, S, heads, d).permute(0, 2, 1, 3)
 
-    q, k, v = r(split(lin("query"))), r(split(lin("key"))), r(split(lin("value")))
+    q, k, v = split(lin("query")), split(lin("key")), split(lin("value"))
     scores = torch.matmul(q, k.transpose(-1, -2)) / math.sqrt(d)
     scores = scores + ext_mask
-    probs = r(torch.softmax(scores, dim=-1))
+    probs = torch.softmax(scores, dim=-1)
     ctx = torch.matmul(probs, v)
-    return r(ctx.permute(0, 2, 1, 3).contiguous().view(B, S, H))
+    return ctx.permute(0, 2, 1, 3).contiguous().view(B, S, H)
 
 
-def layer_torch(x, npy, i, heads, ext_mask, rnd=None, rnd_resid=None):
+def layer_torch(x, npy, i, heads, ext_mask):
     """One BertLayer.                                  modeling.py:256-320"""
     p = f"bert_encoder_layer_{i}_"
-    r = rnd or (lambda t: t)
-    rr = rnd_resid or (lambda t: t)
-    ctx = self_attention_torch(r(x), npy, p, heads, ext_mask, rnd)
-    a = r(ctx @ _t(npy, p + "attention_output_dense_kernel") + _t(npy, p + "attention_output_dense_bias"))
-    x = rr(layer_norm_torch(a + x, _t(npy, p + "attention_output_LayerNorm_gamma"),
-                            _t(npy, p + "attention_output_LayerNorm_beta")))
-    h = r(gelu_torch(r(x) @ _t(npy, p + "intermediate_dense_kernel") + _t(npy, p + "intermediate_dense_bias")))
-    o = r(h @ _t(npy, p + "output_dense_kernel") + _t(npy, p + "output_dense_bias"))
-    return rr(layer_norm_torch(o + x, _t(npy, p + "output_LayerNorm_gamma"),
-                               _t(npy, p + "output_LayerNorm_beta")))
+    ctx = self_attention_torch(x, npy, p, heads, ext_mask)
+    a = ctx @ _t(npy, p + "attention_output_dense_kernel") + _t(npy, p + "attention_output_dense_bias")
+    x = layer_norm_torch(a + x, _t(npy, p + "attention_output_LayerNorm_gamma"),
+                         _t(npy, p + "attention_output_LayerNorm_beta"))
+    h = gelu_torch(x @ _t(npy, p + "intermediate_dense_kernel") + _t(npy, p + "intermediate_dense_bias"))
+    o = h @ _t(npy, p + "output_dense_kernel") + _t(npy, p + "output_dense_bias")
+    return layer_norm_torch(o + x, _t(npy, p + "output_LayerNorm_gamma"),
+                            _t(npy, p + "output_LayerNorm_beta"))
 
 
 def pooler_torch(seq, npy):
@@ -218,43 +214,3 @@ def forward_numpy64(npy, heads: int, ids, seg, mask=None, layers: Optional[int] 
         x = layer_norm_np(o + x, W[p + "output_LayerNorm_gamma"], W[p + "output_LayerNorm_beta"])
     pooled = np.tanh(x[:, 0] @ W["bert_pooler_dense_kernel"] + W["bert_pooler_dense_bias"])
     return x, pooled
-
-
-# --------------------------------------------------------------------------- #
-# Reduced-precision plan emulation (host-side study tool for the tolerance the
-# bf16 engine mode has to meet; not a parity target by itself).
-# --------------------------------------------------------------------------- #
-
-def _round_bf16(t):
-    import torch
-    return t.to(torch.bfloat16).to(torch.float32)
-
-
-def forward_torch_bf16_plan(npy, heads, ids, seg, mask=None, resid_bf16: bool = False):
-    """Emulates: weights and GEMM operands rounded to bf16 (RNE), fp32
-    accumulation, LayerNorm/softmax statistics in fp32, residual stream kept in
-    fp32 (or bf16 when ``resid_bf16``)."""
-    import torch
-    w = {}
-    for k_, v_ in npy.items():
-        a = torch.from_numpy(np.ascontiguousarray(v_))
-        if v_.ndim == 2:
-            a = _round_bf16(a)
-        w[k_] = a.numpy()
-    with torch.no_grad():
-        ids_t = torch.as_tensor(np.asarray(ids), dtype=torch.long)
-        seg_t = torch.as_tensor(np.asarray(seg), dtype=torch.long)
-        mask_t = torch.ones_like(ids_t) if mask is None else torch.as_tensor(np.asarray(mask), dtype=torch.long)
-        ext = extended_mask_torch(mask_t)
-        rr = _round_bf16 if resid_bf16 else None
-        x = embeddings_torch(w, ids_t, seg_t)
-        if rr:
-            x = rr(x)
-        L = 0
-        while f"bert_encoder_layer_{L}_attention_self_query_kernel" in w:
-            L += 1
-        for i in range(L):
-            x = layer_torch(x, w, i, heads, ext, rnd=_round_bf16,
-                            rnd_resid=rr if i + 1 < L else None)
-        pooled = pooler_torch(x, w)
-        return x.numpy(), pooled.numpy()

@@ -154,10 +154,12 @@ def test_cuda_bert_exits_on_error_like_the_reference():
     assert "Cuda_Bert failed" in r.stderr
 
 
-def test_reference_helpers(pb):
-    # cuda_bert/pybert.py:44-60
-    w = pb.filling_inputs([1, 2, 3, 9], 8)
-    assert w == [1, 2, 3, 1, 2, 3, 1, 9]
-    assert pb.filling_inputs(pb.SEED_MASK, 11) == pb.SEED_MASK
-    ids, seg, mask = pb.warp_inputs(pb.batch_inputs(w, 2), pb.batch_inputs(w, 2), pb.batch_inputs(w, 2))
-    assert ids.shape == (2, 8) and ids.dtype == np.int32
+def test_seed_batch(pb):
+    # the stretched seed rows of the reference's benchmarks (cuda_bert/cuda_bert.cu:12-22, 94-103)
+    ids, seg, mask = pb.seed_batch(2, 23)
+    assert ids.shape == seg.shape == mask.shape == (2, 23) and ids.dtype == np.int32
+    assert (ids[0] == ids[1]).all()
+    assert list(ids[0, :10]) == pb.SEED_IDS[:10] and list(ids[0, 10:20]) == pb.SEED_IDS[:10]
+    assert ids[0, -1] == pb.SEED_IDS[-1] and seg[0, -1] == 1 and mask[0, -1] == 0
+    ids11, _, mask11 = pb.seed_batch(1, 11)
+    assert list(ids11[0]) == pb.SEED_IDS and list(mask11[0]) == pb.SEED_MASK

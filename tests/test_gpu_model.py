@@ -30,12 +30,7 @@ def pb():
     return pybert
 
 
-def bf16_exact(state):
-    out = {}
-    for k, v in state.items():
-        t = torch.from_numpy(v)
-        out[k] = t.to(torch.bfloat16).to(torch.float32).numpy() if v.ndim == 2 and "embeddings" not in k else v
-    return out
+bf16_exact = W.bf16_representable
 
 
 def load(pb, dims, wdir, precision, maxB, maxS, graph=0):
