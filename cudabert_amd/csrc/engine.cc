@@ -89,6 +89,7 @@ bool Model::init(const ModelOptions& opt_in) {
         return false;
     }
     CUBERT_HIP_OK(hipSetDevice(opt_.gpu));
+    if (!noalloc_setup_current_device()) return false;
     CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
     for (int i = 1; i < kMaxParts; ++i) {
         CUBERT_HIP_OK(hipStreamCreateWithFlags(&side_[i], hipStreamNonBlocking));

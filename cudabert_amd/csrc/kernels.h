@@ -138,4 +138,8 @@ bool launch_transpose_convert(const float* src, void* dst, int K, int N, int elt
                               hipStream_t stream);
 bool launch_fill_f32(float* dst, float value, size_t n, hipStream_t stream);
 
+// Looks up, for the current device, the address of the scratch array of the allocation-free
+// split-K GEMM (cubert_op_gemm_splitk_noalloc), so that later calls need no symbol lookup.
+bool noalloc_setup_current_device();
+
 }  // namespace cubert

@@ -184,6 +184,21 @@ int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int
 int cubert_op_gemm_residual(const void* X, const void* W, const float* bias, const float* R, float* Y,
                             int M, int N, int K, int ldx, int elt, int tile, int flags, void* stream);
 
+/* Allocation-free split-K GEMM.  No counterpart in the reference: it is for callers that cannot
+ * allocate device memory -- code under hipGraph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Y[M,N] (float32) = X * W^T + bias, K shared by `splits` (1..16) workgroups per tile,
+ * i.e. cubert_op_gemm with epilogue 0, a float32 Y and CUBERT_SPLITS(splits), except that the partial
+ * sums live in a device array built into the library (cubert_noalloc_scratch_bytes() = 16 MiB per GPU,
+ * held until the process ends) and are added up on the device, part 0 first: Y holds M*N floats.
+ * The call makes no hipMalloc / hipFree.  splits * M * N * 4 bytes above the array's size are refused
+ * with an error.  All calls on one GPU share that GPU's array, so calls that overlap in time on one
+ * GPU race; calls on one stream are ordered and need no clearing in between.  The first call on a
+ * device (or creating a model on it) looks the array's address up: make it outside graph capture.
+ * flags: CUBERT_X_PACKED | CUBERT_W_PACKED. */
+int cubert_op_gemm_splitk_noalloc(const void* X, const void* W, const float* bias, float* Y, int M, int N,
+                                  int K, int ldx, int elt, int splits, int tile, int flags, void* stream);
+size_t cubert_noalloc_scratch_bytes(void);
+
 /* Fused QKV projection (op_BatchedLinear::forward, cuda_bert/ops/linear.cu:241-319):
  * X[B*S, hidden] * Wqkv[3*hidden, hidden]^T + bias -> q,k [B,heads,S,64],
  * vt [B,heads,64,Sp] with Sp = S rounded up to 32. */
