@@ -9,9 +9,11 @@ over one synthetic batch of the headline configuration: BERT-large, batch 128,
 seq 200, per-row valid lengths uniform in [100, 200], stock N(0, 0.02) weights.
 Inputs are resident in device memory when the timed region starts.  Prints one
 JSON line with the whole-job rate, the roofline figure of the dominant kernel
-(the FFN GEMM, timed with HIP events around back-to-back launches on the stream
-they are launched on), a per-phase breakdown with achieved TFLOP/s and GB/s,
-and the CPU oracle's rate on a bounded sample of the same batch.
+(the FFN-in GEMM, timed with HIP events on the stream it is launched on), a
+per-phase breakdown with achieved TFLOP/s and GB/s, the stand-alone bandwidth
+kernels, the same pass in float32 operands, the latency regime (batch 1 and 8
+from a hipGraph, p50 / p99), and the CPU oracle's rate on a bounded sample of
+the same batch together with the max-abs difference of the timed pass to it.
 """
 import argparse
 import ctypes
@@ -28,11 +30,23 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 PEAK_HBM_GBS = 8000.0
-# HBM-side bytes of one FFN-in GEMM launch at the headline shape (bf16, packed operands),
-# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --roofline-only`, each
-# counter scaled by what it reads for a 256 MiB device copy (2.0 and 1.0); the summary
-# with the commands is profiles/ffn_in_gemm_cfg2_bf16_pmc.txt.
-MEASURED_TRAFFIC = {("bf16", 25600, 4096, 1024): 6.354e8}
+
+
+def measured_traffic(precision, N, I, H):
+    """HBM-side bytes of one FFN-in GEMM launch at the headline shape, as recorded in
+    profiles/ffn_in_gemm_cfg2_bf16_pmc.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+    `bench.py --roofline-only`, each counter scaled by what it reads for a 256 MiB device copy.
+    The summary names the commit it was measured at; (None, None) for any other shape."""
+    if (precision, N, I, H) != ("bf16", 25600, 4096, 1024):
+        return None, None
+    import re
+    try:
+        text = open(os.path.join(ROOT, "profiles", "ffn_in_gemm_cfg2_bf16_pmc.txt")).read()
+    except OSError:
+        return None, None
+    m = re.search(r"-> traffic ([0-9.e+]+) bytes", text)
+    c = re.search(r"measured at commit ([0-9a-f]+)", text)
+    return (float(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
 def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
@@ -70,18 +84,19 @@ def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
     roofline = {"bound": "mfma", "kernel": "%s (FFN-in %dx%dx%d, tile chosen by the library)" % (kname, N, I, H), "achieved": round(achieved, 1), "peak": PEAK_TFLOPS[precision],
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[precision], 4),
                 "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch,
-                "traffic": MEASURED_TRAFFIC.get((precision, N, I, H))}
+                "traffic": measured_traffic(precision, N, I, H)[0],
+                "traffic_source": "profiles/ffn_in_gemm_cfg2_bf16_pmc.txt (rocprofv3 --pmc, commit %s)" %
+                                  measured_traffic(precision, N, I, H)[1]}
     del X, Wt, Y
     return roofline
 
 
 
-def latency_leg(torch, pybert, synth, model, dims, args):
+def latency_leg(pybert, synth, model, dims, iters, warmup):
     """Config 3: BERT-large, S=200, all positions valid, batch 1 and 8; every call replays the
     captured hipGraph of the whole forward pass.  One call = host inputs in, pooled output
     back on the host (the reference's Cuda_Bert contract), timed with the host clock."""
     lib = pybert.lib
-    iters = max(args.steps, 1000)
     res = {}
     for B in (1, 8):
         S = 200
@@ -89,7 +104,7 @@ def latency_leg(torch, pybert, synth, model, dims, args):
         out = np.empty((B, dims.hidden), np.float32)
         call = lambda: pybert.check(lib.cubert_encode(model, ids.ctypes.data, seg.ctypes.data, mask.ctypes.data, B, S,
                                                       out.ctypes.data, None, None))
-        for _ in range(max(args.warmup, 5)):
+        for _ in range(max(warmup, 5)):
             call()
         ts = np.empty(iters)
         for i in range(iters):
@@ -100,31 +115,22 @@ def latency_leg(torch, pybert, synth, model, dims, args):
                               "p99_ms": round(float(np.percentile(ts, 99)) * 1e3, 4),
                               "mean_ms": round(float(ts.mean()) * 1e3, 4), "iters": iters,
                               "sequences_per_s": round(B / float(ts.mean()), 1)}
-    print(json.dumps({"metric": "latency per batch, BERT-large s200 on 1 MI355X (host in -> host out)", "unit": "ms",
-                      "higher_is_better": False, "n_gpus": 1, "dtype": args.precision, "data": "synthetic",
-                      "config": {"workload": "cfg3: BERT-large encoder + pooler, seq 200 all valid, hipGraph replay",
-                                 "graphs_cached": int(lib.cubert_graphs_cached(model))},
-                      "latency": res}))
+    res["graphs_cached"] = int(lib.cubert_graphs_cached(model))
+    res["what"] = "cfg3: BERT-large s200 all valid, bf16, hipGraph replay; host inputs in -> pooled output on the host"
+    return res
 
 
-def extras_leg(torch, pybert, model, ids, seg, mask, dims, prec, steps):
-    """Host-input entry point (uploads included) and the stand-alone bandwidth-bound kernels."""
+def standalone_ops(torch, pybert, mask, B, S, H, A):
+    """The bandwidth-bound kernels on their own (not inside a pass): residual + LayerNorm as the model
+    launches it in bf16 mode (reads the GEMM result that already holds the residual, writes the float32
+    stream and the packed bf16 copy), the same with the residual read (the reference's cuApplyLayerNorm
+    traffic: 3 float32 passes), and in-place scale + mask + softmax over materialised scores."""
     lib = pybert.lib
-    B, S = ids.shape
-    N, H, A = B * S, dims.hidden, dims.heads
-    out = np.empty((B, H), np.float32)
-    call = lambda: pybert.check(lib.cubert_encode(model, ids.ctypes.data, seg.ctypes.data, mask.ctypes.data, B, S,
-                                                  out.ctypes.data, None, None))
-    for _ in range(2):
-        call()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        call()
-    host_rate = B * steps / (time.perf_counter() - t0)
+    N = B * S
     st = torch.cuda.current_stream()
 
-    def timed(fn, reps=20):
-        for _ in range(3):
+    def timed(fn, reps=30):
+        for _ in range(5):
             fn()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(st)
@@ -134,26 +140,48 @@ def extras_leg(torch, pybert, model, ids, seg, mask, dims, prec, steps):
         e1.synchronize()
         return e0.elapsed_time(e1) / reps
 
+    def entry(ms, by):
+        return {"ms": round(ms, 4), "bytes": by, "gbs": round(by / ms / 1e6, 1),
+                "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
     ops = {}
     x = torch.randn((N, H), device="cuda")
     y = torch.randn((N, H), device="cuda")
     g = torch.ones(H, device="cuda")
     b = torch.zeros(H, device="cuda")
+    xb = torch.empty(((N + 255) // 256 * 256, H), dtype=torch.bfloat16, device="cuda")
     ms = timed(lambda: pybert.check(lib.cubert_op_add_layernorm(x.data_ptr(), y.data_ptr(), 0, g.data_ptr(), b.data_ptr(),
                                                                 None, N, H, 0, st.cuda_stream)))
-    by = 3.0 * N * H * 4 + 2 * H * 4
-    ops["add_layernorm_f32"] = {"ms": round(ms, 4), "bytes": by, "gbs": round(by / ms / 1e6, 1),
-                                "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    ops["add_layernorm_f32"] = entry(ms, 3.0 * N * H * 4 + 2 * H * 4)
+    ops["add_layernorm_f32"]["what"] = "x <- LN(x + y): 2 float32 reads + 1 float32 write per element"
+    ms = timed(lambda: pybert.check(lib.cubert_op_add_layernorm(x.data_ptr(), y.data_ptr(), 0, g.data_ptr(), b.data_ptr(),
+                                                                xb.data_ptr(), N, H, 4 | 16, st.cuda_stream)))
+    ops["layernorm_as_in_bf16_pass"] = entry(ms, (4.0 + 4.0 + 2.0) * N * H + 2 * H * 4)
+    ops["layernorm_as_in_bf16_pass"]["what"] = ("x <- LN(y), residual already added by the GEMM: float32 read + float32 "
+                                                "write + packed bf16 copy per element")
+    dm = torch.from_numpy(mask).cuda()
     for elt, name, tdt, es in ((0, "f32", torch.float32, 4), (1, "bf16", torch.bfloat16, 2)):
         sc = torch.randn((B, A * S, S), device="cuda").to(tdt)
-        dm = torch.from_numpy(mask).cuda()
         ms = timed(lambda: pybert.check(lib.cubert_op_mask_softmax(sc.data_ptr(), elt, dm.data_ptr(), B, A * S, S,
                                                                    0.125, st.cuda_stream)))
-        by = 2.0 * B * A * S * S * es + 4 * B * S
-        ops["mask_softmax_" + name] = {"ms": round(ms, 4), "bytes": by, "gbs": round(by / ms / 1e6, 1),
-                                       "frac_hbm_peak": round(by / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        ops["mask_softmax_" + name] = entry(ms, 2.0 * B * A * S * S * es + 4 * B * S)
         del sc
-    return {"host_inputs_sequences_per_s": round(host_rate, 1), "ops": ops}
+    return ops
+
+
+def host_input_rate(pybert, model, ids, seg, mask, H, steps):
+    """Host-input entry point: uploads and the pooled-output download are inside the timed region."""
+    lib = pybert.lib
+    B, S = ids.shape
+    out = np.empty((B, H), np.float32)
+    call = lambda: pybert.check(lib.cubert_encode(model, ids.ctypes.data, seg.ctypes.data, mask.ctypes.data, B, S,
+                                                  out.ctypes.data, None, None))
+    for _ in range(2):
+        call()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    return round(B * steps / (time.perf_counter() - t0), 1)
 
 
 def main():
@@ -164,9 +192,10 @@ def main():
     ap.add_argument("--precision", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4],
                     help="2 = headline; 3 = latency regime (B=1 and 8, hipGraph replay, p50/p99)")
-    ap.add_argument("--extras", action="store_true",
-                    help="also time the host-input entry point (PCIe inclusive) and the stand-alone "
-                         "bandwidth-bound kernels (residual+LayerNorm, scale+mask+softmax, embedding+LayerNorm)")
+    ap.add_argument("--extras", action="store_true", help="also time the host-input entry point (PCIe inclusive)")
+    ap.add_argument("--no-side-legs", action="store_true",
+                    help="config 2 only: skip the pass in the other precision and the latency regime (cfg3) "
+                         "that the default run records beside the headline figure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seqs", type=int, default=128, help="sequences in the CPU baseline sample")
     ap.add_argument("--graph", action="store_true", help="replay the whole pass from a hipGraph (as small batches do by default)")
@@ -212,38 +241,105 @@ def main():
     state = W.synth_state(dims, seed=20240, degenerate=True)
     npy = W.to_npy_layout(state)
     del state
-    with tempfile.TemporaryDirectory(prefix="cubert_w_") as wdir:
-        for name, arr in npy.items():
-            np.save(os.path.join(wdir, name + ".npy"), arr)
-        t_gen = time.time() - t0
-        t0 = time.time()
-        model = pybert.load_model_ex(wdir, H, L, A, I, precision=prec, max_batchsize=B, max_seq_length=S,
-                                     graph_max_tokens=8192 if args.config == 3 else (1 << 30 if args.graph else 0))
-        t_load = time.time() - t0
+    wtmp = tempfile.TemporaryDirectory(prefix="cubert_w_")
+    wdir = wtmp.name
+    for name, arr in npy.items():
+        np.save(os.path.join(wdir, name + ".npy"), arr)
+    t_gen = time.time() - t0
+    t0 = time.time()
+    model = pybert.load_model_ex(wdir, H, L, A, I, precision=prec, max_batchsize=B, max_seq_length=S,
+                                 graph_max_tokens=8192 if args.config == 3 else (1 << 30 if args.graph else 0))
+    t_load = time.time() - t0
     lib = pybert.lib
     if args.config == 3:
-        latency_leg(torch, pybert, synth, model, dims, args)
+        lat = latency_leg(pybert, synth, model, dims, max(args.steps, 1000), args.warmup)
         pybert.unload_model(model)
+        wtmp.cleanup()
+        print(json.dumps({"metric": "latency per batch, BERT-large s200 on 1 MI355X (host in -> host out)", "unit": "ms",
+                          "higher_is_better": False, "n_gpus": 1, "dtype": args.precision, "data": "synthetic",
+                          "config": {"workload": lat["what"]}, "latency": lat}))
         return
     d_ids, d_seg, d_mask = (torch.from_numpy(a).cuda() for a in (ids, seg, mask))
     torch.cuda.synchronize()
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
 
-    def step():
-        pybert.check(lib.cubert_forward_device(model, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S))
-        pybert.check(lib.cubert_classify(model))
+    def timed_pass(mdl, steps, warmup):
+        def step():
+            pybert.check(lib.cubert_forward_device(mdl, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S))
+            pybert.check(lib.cubert_classify(mdl))
+        for _ in range(warmup):
+            step()
+        pybert.check(lib.cubert_sync(mdl))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        pybert.check(lib.cubert_sync(mdl))
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
 
-    for _ in range(args.warmup):
-        step()
-    pybert.check(lib.cubert_sync(model))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    pybert.check(lib.cubert_sync(model))
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    def results_of(mdl):
+        """Sequence and pooled output of the last pass, copied to the host."""
+        pybert.check(lib.cubert_sync(mdl))
+        pooled = np.empty((B, H), np.float32)
+        seq = np.empty((B, S, H), np.float32)
+        assert hip.hipMemcpy(pooled.ctypes.data, lib.cubert_pooled_ptr(mdl), pooled.nbytes, 2) == 0
+        assert hip.hipMemcpy(seq.ctypes.data, lib.cubert_seq_ptr(mdl), seq.nbytes, 2) == 0
+        return seq, pooled
+
+    def phase_profile(mdl, precision_name, reps=3):
+        """Per-phase breakdown: one event before every launch of an eager single-stream pass."""
+        e = 2 if precision_name == "bf16" else 4
+        ph = (ctypes.c_float * 8)()
+        acc = np.zeros(8)
+        for _ in range(reps):
+            pybert.check(lib.cubert_profile_device(mdl, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S, ph))
+            acc += np.array(list(ph))
+        acc /= reps
+        gf = {"qkv_gemm": 2.0 * N * H * 3 * H * L, "attn_out_gemm": 2.0 * N * H * H * L,
+              "ffn_in_gemm": 2.0 * N * H * I * L, "ffn_out_gemm": 2.0 * N * I * H * L,
+              "attention": 4.0 * N * S * H * L, "pooler": 2.0 * B * H * H}
+        Sp = (S + 31) // 32 * 32
+        # residual+LayerNorm, algorithmic: x read + y read + x write, float32 (the reference's kernel)
+        ln_bytes_alg = (3.0 * N * H * 4 + 2 * H * 4) * 2 * L
+        # bytes the LayerNorm kernel itself moves: the residual is added by the GEMM before it (unless
+        # CUBERT_FUSE_RESIDUAL=0), so it reads the sum and writes the float32 stream (+ the bf16 copy)
+        ln_reads = 1 if os.environ.get("CUBERT_FUSE_RESIDUAL", "1") != "0" else 2
+        ln_bytes_exec = (((ln_reads + 1) * 4 + (2 if e == 2 else 0)) * N * H + 2 * H * 4) * 2 * L
+        emb_bytes = N * (12 + H * 4 + H * 4) + (S + 2) * H * 4 + 2 * H * 4
+        # fused attention reads q, k, v^T and the mask rows and writes the context: its HBM bytes
+        att_bytes = ((3.0 * N * H + 1.0 * N * H) * e + B * A * 64 * (Sp - S) * e + 4.0 * B * Sp) * L
+        phases = {}
+        for i, name in enumerate(pybert.PHASES):
+            ms = float(acc[i])
+            d = {"ms": round(ms, 4)}
+            if name in gf and ms > 0:
+                d["tflops"] = round(gf[name] / ms / 1e9, 1)
+                d["frac_mfma_peak"] = round(d["tflops"] / PEAK_TFLOPS[precision_name], 4)
+            if name == "add_layernorm" and ms > 0:
+                d["gbs_algorithmic"] = round(ln_bytes_alg / ms / 1e6, 1)
+                d["gbs_executed"] = round(ln_bytes_exec / ms / 1e6, 1)
+                d["frac_hbm_peak_executed"] = round(d["gbs_executed"] / PEAK_HBM_GBS, 4)
+                d["frac_hbm_peak_algorithmic"] = round(d["gbs_algorithmic"] / PEAK_HBM_GBS, 4)
+            if name == "attention" and ms > 0:
+                # S = 200: 97 FLOP per byte, below the machine balance (312), so HBM is the roof
+                d["bound"] = "hbm"
+                d["gbs"] = round(att_bytes / ms / 1e6, 1)
+                d["frac_hbm_peak"] = round(d["gbs"] / PEAK_HBM_GBS, 4)
+            if name == "embedding" and ms > 0:
+                d["gbs_algorithmic"] = round(emb_bytes / ms / 1e6, 1)
+            phases[name] = d
+        gemm_ms = sum(acc[i] for i, n in enumerate(pybert.PHASES) if n.endswith("_gemm"))
+        gemm_flops = sum(gf[n] for n in gf if n.endswith("_gemm"))
+        phases["all_gemms"] = {"ms": round(float(gemm_ms), 3), "tflops": round(gemm_flops / gemm_ms / 1e9, 1),
+                               "frac_mfma_peak": round(gemm_flops / gemm_ms / 1e9 / PEAK_TFLOPS[precision_name], 4)}
+        return phases, float(acc[pybert.PHASES.index("ffn_in_gemm")]) / L, gemm_flops
+
+    elapsed = timed_pass(model, args.steps, args.warmup)
     ms_per_step = elapsed * 1e3 / args.steps
     value = B * args.steps / elapsed
+    seq_gpu, pooled_gpu = results_of(model)
 
     # ---- the same batch computed on its valid tokens only (not the headline figure: the padded
     # pass above also fills the padding positions of the sequence output, as the reference does) ----
@@ -266,43 +362,7 @@ def main():
                 "note": "cubert_forward_device_lens: only valid tokens computed; pooled output and valid "
                         "positions bit-identical to the padded pass"}
 
-    # ---- per-phase breakdown (events before every launch; outside the timed region) ----
-    ph = (ctypes.c_float * 8)()
-    acc = np.zeros(8)
-    reps = 3
-    for _ in range(reps):
-        pybert.check(lib.cubert_profile_device(model, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S, ph))
-        acc += np.array(list(ph))
-    acc /= reps
-    gf = {"qkv_gemm": 2.0 * N * H * 3 * H * L, "attn_out_gemm": 2.0 * N * H * H * L,
-          "ffn_in_gemm": 2.0 * N * H * I * L, "ffn_out_gemm": 2.0 * N * I * H * L,
-          "attention": 4.0 * N * S * H * L, "pooler": 2.0 * B * H * H}
-    # residual+LayerNorm traffic as executed: x f32 read + y f32 read + x f32 write (+ bf16 copy)
-    ln_bytes_alg = (3.0 * N * H * 4 + 2 * H * 4) * 2 * L
-    # bytes the LayerNorm kernel itself moves: the residual is added by the GEMM before it (unless
-    # CUBERT_FUSE_RESIDUAL=0), so it reads the sum and writes the float32 stream (+ the bf16 copy)
-    ln_reads = 1 if os.environ.get("CUBERT_FUSE_RESIDUAL", "1") != "0" else 2
-    ln_bytes_exec = (((ln_reads + 1) * 4 + (2 if prec == pybert.BF16 else 0)) * N * H + 2 * H * 4) * 2 * L
-    emb_bytes = N * (12 + H * 4 + H * 4) + (S + 2) * H * 4 + 2 * H * 4
-    phases = {}
-    for i, name in enumerate(pybert.PHASES):
-        ms = float(acc[i])
-        e = {"ms": round(ms, 4)}
-        if name in gf and ms > 0:
-            e["tflops"] = round(gf[name] / ms / 1e9, 1)
-            e["frac_mfma_peak"] = round(e["tflops"] / PEAK_TFLOPS[args.precision], 4)
-        if name == "add_layernorm" and ms > 0:
-            e["gbs_algorithmic"] = round(ln_bytes_alg / ms / 1e6, 1)
-            e["gbs_executed"] = round(ln_bytes_exec / ms / 1e6, 1)
-            e["frac_hbm_peak_executed"] = round(e["gbs_executed"] / PEAK_HBM_GBS, 4)
-            e["frac_hbm_peak_algorithmic"] = round(e["gbs_algorithmic"] / PEAK_HBM_GBS, 4)
-        if name == "embedding" and ms > 0:
-            e["gbs_algorithmic"] = round(emb_bytes / ms / 1e6, 1)
-        phases[name] = e
-    gemm_ms = sum(acc[i] for i, n in enumerate(pybert.PHASES) if n.endswith("_gemm"))
-    gemm_flops = sum(gf[n] for n in gf if n.endswith("_gemm"))
-    phases["all_gemms"] = {"ms": round(float(gemm_ms), 3), "tflops": round(gemm_flops / gemm_ms / 1e9, 1),
-                           "frac_mfma_peak": round(gemm_flops / gemm_ms / 1e9 / PEAK_TFLOPS[args.precision], 4)}
+    phases, k_ms, gemm_flops = phase_profile(model, args.precision)
 
     # The roofline entry is the FFN-in GEMM as it runs inside the forward pass: HIP events on the launch
     # stream around each of its L launches, averaged over the passes above.  The stand-alone leg (50
@@ -310,14 +370,41 @@ def main():
     # kept beside it.
     standalone = roofline_leg(torch, pybert, lib, prec, args.precision, N, I, H)
     roofline = dict(standalone)
-    k_ms = float(acc[pybert.PHASES.index("ffn_in_gemm")]) / L
     if k_ms > 0:
         achieved = standalone["flop_per_launch"] / k_ms / 1e9
         roofline.update({"achieved": round(achieved, 1), "frac": round(achieved / PEAK_TFLOPS[args.precision], 4),
                          "avg_launch_ms": round(k_ms, 4),
-                         "measured": "HIP events around each of the %d FFN-in launches of a forward pass, %d passes" % (L, reps),
+                         "measured": "HIP events around each of the %d FFN-in launches of a forward pass, 3 passes" % L,
                          "standalone_back_to_back": {"launches": 50, "avg_launch_ms": standalone["avg_launch_ms"],
                                                      "achieved": standalone["achieved"], "frac": standalone["frac"]}})
+    ops = standalone_ops(torch, pybert, mask, B, S, H, A)
+    host_rate = host_input_rate(pybert, model, ids, seg, mask, H, args.steps) if args.extras else None
+    pybert.unload_model(model)
+
+    # ---- the other precision of the same configuration, and the latency regime, in the same record ----
+    other_pass = latency = None
+    seq_other = pooled_other = None
+    if args.config == 2 and not args.no_side_legs:
+        oname = "fp32" if args.precision == "bf16" else "bf16"
+        oprec = pybert.F32 if oname == "fp32" else pybert.BF16
+        m2 = pybert.load_model_ex(wdir, H, L, A, I, precision=oprec, max_batchsize=B, max_seq_length=S, graph_max_tokens=0)
+        osteps = 5 if oname == "fp32" else args.steps
+        dt = timed_pass(m2, osteps, 2)
+        seq_other, pooled_other = results_of(m2)
+        oph, ok_ms, oflops = phase_profile(m2, oname, reps=1 if oname == "fp32" else 3)
+        other_pass = {"dtype": oname, "value": round(B * osteps / dt, 2), "unit": "sequences/s", "steps": osteps,
+                      "ms_per_step": round(dt * 1e3 / osteps, 3),
+                      "roofline": {"bound": "mfma", "kernel": "FFN-in GEMM %dx%dx%d inside the forward pass" % (N, I, H),
+                                   "achieved": round(2.0 * N * H * I / ok_ms / 1e9, 1), "peak": PEAK_TFLOPS[oname],
+                                   "unit": "TFLOP/s", "frac": round(2.0 * N * H * I / ok_ms / 1e9 / PEAK_TFLOPS[oname], 4),
+                                   "avg_launch_ms": round(ok_ms, 4)},
+                      "phases": oph}
+        pybert.unload_model(m2)
+        m3 = pybert.load_model_ex(wdir, H, L, A, I, precision=pybert.BF16, max_batchsize=8, max_seq_length=200,
+                                  graph_max_tokens=8192)
+        latency = latency_leg(pybert, synth, m3, dims, 1000, 10)
+        pybert.unload_model(m3)
+    wtmp.cleanup()
 
     # ---- CPU baseline: the oracle on a bounded sample of the same batch ----
     cpu = None
@@ -333,16 +420,14 @@ def main():
         dt = time.perf_counter() - t0
         cpu = {"value": round(n / dt, 3), "unit": "sequences/s", "cores": cores, "kind": "port",
                "sample": "first %d sequences of the same batch (S=%d), fp32 torch oracle, 1 pass, %.1f s" % (n, S, dt)}
-        # the sample doubles as a full-size parity spot check
-        pooled = torch.empty((B, H), device="cuda")
-        hip = ctypes.CDLL("libamdhip64.so")
-        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
-        step()
-        pybert.check(lib.cubert_sync(model))
-        assert hip.hipMemcpy(pooled.data_ptr(), lib.cubert_pooled_ptr(model), B * H * 4, 3) == 0
-        cpu["pooled_max_abs_vs_gpu"] = float(np.abs(pooled.cpu().numpy()[:n] - pooled_ref).max())
-    extras = extras_leg(torch, pybert, model, ids, seg, mask, dims, prec, args.steps) if args.extras else None
-    pybert.unload_model(model)
+        # The sample doubles as a full-size parity check of the timed pass (float32 oracle on the
+        # unrounded checkpoint; in bf16 mode the error includes rounding the weights to bfloat16).
+        cpu["pooled_max_abs_vs_gpu"] = float(np.abs(pooled_gpu[:n] - pooled_ref).max())
+        cpu["seq_max_abs_vs_gpu"] = float(np.abs(seq_gpu[:n] - seq_ref).max())
+        cpu["seq_rms_vs_gpu"] = float(np.sqrt(np.mean((seq_gpu[:n] - seq_ref) ** 2, dtype=np.float64)))
+        if other_pass is not None:
+            other_pass["pooled_max_abs_vs_cpu"] = float(np.abs(pooled_other[:n] - pooled_ref).max())
+            other_pass["seq_max_abs_vs_cpu"] = float(np.abs(seq_other[:n] - seq_ref).max())
 
     out = {
         "metric": "sequences/s BERT-large b128 s200 on 1 MI355X" if args.config == 2 else
@@ -355,11 +440,16 @@ def main():
                                (args.config, "large" if large else "base", B, S),
                    "batch": B, "seq_len": S, "tokens": N, "precision": args.precision},
         "roofline": roofline, "cpu_baseline": cpu, "unpadded_pass": unpadded, "phases": phases,
+        "standalone_ops": ops,
         "gemm_tflop_per_step": round(gemm_flops / 1e12, 3),
         "setup_s": {"weights_generate_write": round(t_gen, 1), "model_load": round(t_load, 1)},
     }
-    if extras:
-        out["extras"] = extras
+    if other_pass is not None:
+        out["%s_pass" % other_pass["dtype"]] = other_pass
+    if latency is not None:
+        out["latency"] = latency
+    if host_rate is not None:
+        out["host_inputs_sequences_per_s"] = host_rate
     print(json.dumps(out))
 
 
