@@ -169,6 +169,109 @@ def standalone_ops(torch, pybert, mask, B, S, H, A):
     return ops
 
 
+class PowerSampler:
+    """Reads the socket power (hwmon power1_input, microwatts) and the shader clock (the starred
+    level of pp_dpm_sclk) of card 0 every few milliseconds in a thread while a workload runs.
+    Read-only sysfs files; entries are None when the box does not expose them."""
+
+    HWMON = "/sys/class/drm/card0/device/hwmon"
+    SCLK = "/sys/class/drm/card0/device/pp_dpm_sclk"
+
+    def __init__(self):
+        self.power_file = None
+        try:
+            for h in sorted(os.listdir(self.HWMON)):
+                f = os.path.join(self.HWMON, h, "power1_input")
+                if os.path.exists(f):
+                    self.power_file = f
+                    self.cap_file = os.path.join(self.HWMON, h, "power1_cap")
+        except OSError:
+            pass
+
+    def _read(self):
+        try:
+            p = int(open(self.power_file).read()) / 1e6
+            star = [l for l in open(self.SCLK).read().splitlines() if "*" in l]
+            mhz = float(star[0].split(":")[1].strip().lower().split("mhz")[0]) if star else None
+            return p, mhz
+        except (OSError, ValueError, IndexError):
+            return None, None
+
+    def measure(self, fn, seconds):
+        """Calls fn() repeatedly for `seconds`; returns average power / clock over the run's later 80 %."""
+        import threading
+        if not self.power_file:
+            return None
+        samples, stop = [], threading.Event()
+
+        def loop():
+            while not stop.is_set():
+                samples.append((time.perf_counter(),) + self._read())
+                time.sleep(0.004)
+        th = threading.Thread(target=loop, daemon=True)
+        th.start()
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < seconds:
+            fn()
+            n += 1
+        t1 = time.perf_counter()
+        stop.set()
+        th.join()
+        sel = [(p, c) for t, p, c in samples if t0 + 0.2 * (t1 - t0) <= t <= t1 and p is not None]
+        if not sel:
+            return None
+        try:
+            cap = int(open(self.cap_file).read()) / 1e6
+        except (OSError, ValueError):
+            cap = None
+        clocks = [c for _, c in sel if c is not None]
+        return {"power_w": round(sum(p for p, _ in sel) / len(sel), 1), "power_cap_w": cap,
+                "sclk_mhz": round(sum(clocks) / len(clocks), 1) if clocks else None,
+                "ms_per_call": round((t1 - t0) * 1e3 / n, 4), "samples": len(sel)}
+
+
+def power_leg(torch, pybert, lib, step, sync, prec, N, I, H):
+    """Where the pass stands against the board's power limit: socket power and shader clock during
+    the forward pass, and during the FFN-in GEMM on its own with the pass's kind of data (random)
+    and with all-zero operands (no data toggling: the same schedule at the full clock)."""
+    ps = PowerSampler()
+    if not ps.power_file:
+        return None
+    out = {}
+
+    def passes():
+        for _ in range(5):
+            step()
+        sync()
+    out["forward_pass"] = ps.measure(passes, 2.0)
+    if out["forward_pass"]:
+        out["forward_pass"]["ms_per_pass"] = round(out["forward_pass"].pop("ms_per_call") / 5, 3)
+    if prec != pybert.BF16:
+        return out
+    st = torch.cuda.current_stream()
+    rows = (N + 255) // 256 * 256
+    bias = torch.zeros(I, device="cuda")
+    Y = torch.empty((rows, I), dtype=torch.bfloat16, device="cuda")
+    for name, zero in (("ffn_in_gemm_random_operands", False), ("ffn_in_gemm_zero_operands", True)):
+        X = (torch.zeros if zero else torch.randn)((rows, H), device="cuda").to(torch.bfloat16)
+        Wt = ((torch.zeros if zero else torch.randn)((I, H), device="cuda") * 0.02).to(torch.bfloat16)
+
+        def launches():
+            for _ in range(40):
+                pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H,
+                                                1, 1, 1, 0, 7, st.cuda_stream))
+            torch.cuda.synchronize()
+        r = ps.measure(launches, 1.5)
+        if r:
+            ms = r.pop("ms_per_call") / 40
+            r["avg_launch_ms"] = round(ms, 4)
+            r["tflops"] = round(2.0 * N * H * I / ms / 1e9, 1)
+            r["frac_mfma_peak"] = round(r["tflops"] / PEAK_TFLOPS["bf16"], 4)
+        out[name] = r
+    return out
+
+
 def host_input_rate(pybert, model, ids, seg, mask, H, steps):
     """Host-input entry point: uploads and the pooled-output download are inside the timed region."""
     lib = pybert.lib
@@ -194,8 +297,8 @@ def main():
                     help="2 = headline; 3 = latency regime (B=1 and 8, hipGraph replay, p50/p99)")
     ap.add_argument("--extras", action="store_true", help="also time the host-input entry point (PCIe inclusive)")
     ap.add_argument("--no-side-legs", action="store_true",
-                    help="config 2 only: skip the pass in the other precision and the latency regime (cfg3) "
-                         "that the default run records beside the headline figure")
+                    help="skip what the default run records beside the headline figure: the pass in the other "
+                         "precision and the latency regime (config 2 only), power and clock sampling")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seqs", type=int, default=128, help="sequences in the CPU baseline sample")
     ap.add_argument("--graph", action="store_true", help="replay the whole pass from a hipGraph (as small batches do by default)")
@@ -378,6 +481,12 @@ def main():
                          "standalone_back_to_back": {"launches": 50, "avg_launch_ms": standalone["avg_launch_ms"],
                                                      "achieved": standalone["achieved"], "frac": standalone["frac"]}})
     ops = standalone_ops(torch, pybert, mask, B, S, H, A)
+
+    def one_pass():
+        pybert.check(lib.cubert_forward_device(model, d_ids.data_ptr(), d_seg.data_ptr(), d_mask.data_ptr(), B, S))
+        pybert.check(lib.cubert_classify(model))
+    power = None if args.no_side_legs else power_leg(torch, pybert, lib, one_pass, lambda: pybert.check(lib.cubert_sync(model)),
+                                                     prec, N, I, H)
     host_rate = host_input_rate(pybert, model, ids, seg, mask, H, args.steps) if args.extras else None
     pybert.unload_model(model)
 
@@ -448,6 +557,8 @@ def main():
         out["%s_pass" % other_pass["dtype"]] = other_pass
     if latency is not None:
         out["latency"] = latency
+    if power is not None:
+        out["power"] = power
     if host_rate is not None:
         out["host_inputs_sequences_per_s"] = host_rate
     print(json.dumps(out))
