@@ -330,14 +330,42 @@ def main():
     es = 2 if prec == pybert.BF16 else 4
 
     if args.roofline_only:
+        # For profiler runs (rocprofv3 --pmc / --kernel-trace): the dominant GEMM, the two bandwidth-bound
+        # kernels of the pass at this configuration's shapes, and one device copy of known size.
         lib = pybert.lib
         roofline = roofline_leg(torch, pybert, lib, prec, args.precision, N, I, H)
+        st = torch.cuda.current_stream()
+        tdt = torch.bfloat16 if prec == pybert.BF16 else torch.float32
+        rows = (N + 255) // 256 * 256
+        # residual + LayerNorm as the pass launches it: reads the GEMM result, writes the float32 stream
+        # (+ the packed bf16 copy in bf16 mode)
+        x = torch.randn((N, H), device="cuda")
+        y = torch.randn((N, H), device="cuda")
+        g, b = torch.ones(H, device="cuda"), torch.zeros(H, device="cuda")
+        xb = torch.empty((rows, H), dtype=torch.bfloat16, device="cuda")
+        for _ in range(20):
+            pybert.check(lib.cubert_op_add_layernorm(x.data_ptr(), y.data_ptr(), 0, g.data_ptr(), b.data_ptr(),
+                                                     xb.data_ptr() if prec == pybert.BF16 else None, N, H,
+                                                     (4 if prec == pybert.BF16 else 0) | 16, st.cuda_stream))
+        # fused attention on this configuration's ragged masks
+        Sp = (S + 31) // 32 * 32
+        q = torch.randn((B, A, S, 64), device="cuda").to(tdt)
+        k = torch.randn((B, A, S, 64), device="cuda").to(tdt)
+        vt = torch.randn((B, A, 64, Sp), device="cuda").to(tdt)
+        madd = np.full((B, Sp), -np.inf, np.float32)
+        madd[:, :S] = (1.0 - mask.astype(np.float32)) * -10000.0
+        madd = torch.from_numpy(madd).cuda()
+        ctx = torch.empty((rows, H), dtype=tdt, device="cuda")
+        for _ in range(20):
+            pybert.check(lib.cubert_op_attention(q.data_ptr(), k.data_ptr(), vt.data_ptr(), madd.data_ptr(), ctx.data_ptr(),
+                                                 B, A, S, 0.125, prec, 4 if prec == pybert.BF16 else 0, st.cuda_stream))
         a = torch.empty(64 << 20, dtype=torch.float32, device="cuda")     # 256 MiB read + 256 MiB written
-        b = torch.empty_like(a)
+        c = torch.empty_like(a)
         for _ in range(3):
-            b.copy_(a)
+            c.copy_(a)
         torch.cuda.synchronize()
-        print(json.dumps({"roofline": roofline, "calibration_copy_bytes_each_way": a.numel() * 4}))
+        print(json.dumps({"roofline": roofline, "calibration_copy_bytes_each_way": a.numel() * 4,
+                          "layernorm_launches": 20, "attention_launches": 20}))
         return
 
     t0 = time.time()
