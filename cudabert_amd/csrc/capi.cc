@@ -55,7 +55,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.graph_cache = env_int("CUBERT_GRAPH_CACHE", 64);
     opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
     opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
-    opt.varlen = env_int("CUBERT_VARLEN", 0) != 0;
+    opt.varlen = env_int("CUBERT_VARLEN", -1);
     opt.split_k = env_int("CUBERT_SPLIT_K", 1) != 0;
     opt.fuse_residual = env_int("CUBERT_FUSE_RESIDUAL", 1) != 0;
     opt.gpu = gpu;
@@ -115,7 +115,7 @@ int cubert_encode(void* model, const int* words, const int* token_types, const i
     cubert::set_error("");
     Model* m = as_model(model, "cubert_encode");
     if (!m) return 1;
-    if (!m->forward_host(words, token_types, attention_mask, batchsize, seq_length)) return 1;
+    if (!m->forward_host(words, token_types, attention_mask, batchsize, seq_length, seq_out != nullptr)) return 1;
     if (cls_out && !m->classify()) return 1;
     if (pooled_out && !m->copy_pooled(pooled_out)) return 1;
     if (seq_out && !m->copy_seq(seq_out)) return 1;

@@ -242,7 +242,7 @@ bool Model::check_shape(int B, int S) {
     return true;
 }
 
-bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B, int S) {
+bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B, int S, bool need_seq) {
     if (!check_shape(B, S)) return false;
     if (!ids || !seg) { set_error("input_ids and token_type_ids must not be null"); return false; }
     const size_t n = (size_t)B * S, cap = (size_t)cap_tokens_;
@@ -266,10 +266,16 @@ bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B,
     CUBERT_HIP_OK(hipMemcpyAsync(d_in_, h_in_, n * 4, hipMemcpyHostToDevice, stream_));
     CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + cap, h_in_ + cap, n * 4, hipMemcpyHostToDevice, stream_));
     if (mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, h_in_ + 2 * cap, n * 4, hipMemcpyHostToDevice, stream_));
-    if (opt_.varlen && mask) {
-        // masks that are 1 on a non-empty prefix and 0 after it: compute the valid tokens only
+    // Masks that are 1 on a non-empty prefix and 0 after it allow the unpadded pass (valid tokens
+    // only; same pooled output bit for bit, zeros instead of values on the padding positions of the
+    // sequence output).  varlen = 1: whenever the masks allow it.  varlen = -1 (default): only when
+    // the caller cannot see the sequence output, the batch is too large for hipGraph replay and at
+    // least 5 % of it is padding.
+    const bool too_big_for_graph = opt_.graph_max_tokens <= 0 || (long)n > opt_.graph_max_tokens;
+    if (mask && (opt_.varlen == 1 || (opt_.varlen < 0 && !need_seq && too_big_for_graph))) {
         std::vector<int> lens(B);
         bool prefix = true;
+        size_t valid = 0;
         for (int b = 0; b < B && prefix; ++b) {
             const int* m = mask + (size_t)b * S;
             int len = 0;
@@ -277,8 +283,9 @@ bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B,
             for (int s = len; s < S && prefix; ++s) prefix = m[s] == 0;
             prefix = prefix && len >= 1;
             lens[b] = len;
+            valid += (size_t)len;
         }
-        if (prefix) return run_compact(lens.data(), B, S);
+        if (prefix && (opt_.varlen == 1 || valid * 20 <= n * 19)) return run_compact(lens.data(), B, S);
     }
     return run(B, S, mask != nullptr);
 }

@@ -28,7 +28,8 @@ struct ModelOptions {
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
     bool fuse_residual = true;     // residual add in the epilogue of the GEMM before each LayerNorm
     bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
-    bool varlen = false;           // host-input calls with prefix masks compute only the valid tokens
+    int varlen = -1;               // host-input calls with prefix masks compute only the valid tokens: 1 always,
+                                   // 0 never, -1 when the caller asks for no sequence output (see forward_host)
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
     int graph_cache = 64;          // instantiated hipGraphs kept per model (least recently used is dropped)
     std::string dir;
@@ -46,7 +47,8 @@ class Model {
     ~Model();
 
     // Host inputs [B, S] int32 (mask may be nullptr).  Asynchronous.
-    bool forward_host(const int* ids, const int* seg, const int* mask, int B, int S);
+    // need_seq: the caller will read the sequence output (else only pooled / classifier results).
+    bool forward_host(const int* ids, const int* seg, const int* mask, int B, int S, bool need_seq = true);
     // Inputs already in device memory.  Asynchronous on stream().
     bool forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S);
     // Unpadded forward: only the first h_lens[b] >= 1 tokens of every sequence are computed (as if

@@ -120,9 +120,15 @@ int cubert_sync(void* model);
  * The pooled output and the sequence output on the valid positions are bit-identical
  * to cubert_forward_device with the corresponding prefix mask; the sequence output is
  * zero on the padding positions (the padded pass computes values there that no caller
- * uses).  The host-input entry points (Cuda_Bert, Cuda_Inference, cubert_encode) take
- * this path by themselves when CUBERT_VARLEN=1 and every mask row is a non-empty
- * prefix of ones.  Returns 0 on success. */
+ * uses).  The host-input entry points take this path by themselves when every mask row
+ * is a non-empty prefix of ones and
+ *   CUBERT_VARLEN=1:      always (Cuda_Bert, Cuda_Classify, Cuda_Inference, cubert_encode);
+ *   CUBERT_VARLEN unset:  only for calls that return no sequence output (Cuda_Bert,
+ *                         Cuda_Classify, cubert_encode with seq_out == NULL), on batches above
+ *                         the hipGraph limit with at least 5 % padding -- the results such a
+ *                         call returns are bit-identical either way;
+ *   CUBERT_VARLEN=0:      never.
+ * Returns 0 on success. */
 int cubert_forward_device_lens(void* model, const int* d_words, const int* d_token_types,
                                const int* lengths, int batchsize, int seq_length);
 

@@ -249,6 +249,44 @@ def test_unpadded_pass_against_the_oracle(pb, tmp_path, precision):
         pb.unload_model(m)
 
 
+def test_pooled_only_host_calls_compute_valid_tokens_only(pb, tmp_path, monkeypatch):
+    """Cuda_Bert / Cuda_Classify return no sequence output, so on a ragged batch they take the
+    unpadded pass by themselves; what they return equals the padded pass bit for bit.  A call
+    that asks for the sequence output stays on the padded pass (values on the padding positions
+    as the PyTorch model defines them)."""
+    D = W.TINY
+    state = W.bf16_representable(W.synth_state(D, seed=21, degenerate=False))
+    wdir = W.export_npy_dir(state, str(tmp_path / "w"))
+    npy = W.to_npy_layout(state)
+    B, S = 5, 40
+    ids, seg, mask = synth.make_inputs(B, S, [40, 3, 17, 1, 22], vocab=D.vocab, seed=3, prune=False)
+    seq_ref, pooled_ref = O.forward_torch(npy, D.heads, ids, seg, mask)
+    monkeypatch.setenv("CUBERT_SPLIT_K", "0")      # split K would group the sums by the row count
+    for precision in (F32, BF16):
+        m = load(pb, D, wdir, precision, B, S)
+        try:
+            pooled_full, seq_full, cls_full = pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)
+            assert err(seq_full, seq_ref) < TOL[precision]          # padded pass: every position defined
+            out = np.ones((B, D.hidden), np.float32)
+            pb.bert(m, out, ids, seg, B, S, mask)
+            assert np.array_equal(out, pooled_full)
+            # the sequence buffer of that call holds zeros on the padding: the unpadded pass ran
+            _, seq_dev = device_results(pb, m, B, S, D.hidden)
+            valid = mask.astype(bool)
+            assert (seq_dev[~valid] == 0).all() and np.array_equal(seq_dev[valid], seq_full[valid])
+            probs = np.zeros((B, 2), np.float32)
+            pb.classify(m, probs, ids, seg, B, S, 2, mask)
+            assert np.array_equal(probs, cls_full)
+            # all-valid batches and masks with holes stay on the padded pass
+            holed = mask.copy()
+            holed[0, 5] = 0
+            pb.bert(m, out, ids, seg, B, S, holed)
+            _, seq_dev = device_results(pb, m, B, S, D.hidden)
+            assert (seq_dev[~valid] != 0).any()
+        finally:
+            pb.unload_model(m)
+
+
 # ------------------------------------------------------------------ hipGraph cache ----
 
 def test_graph_cache_keeps_shapes_apart_beyond_1024_positions(pb, tmp_path):
