@@ -58,6 +58,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.varlen = env_int("CUBERT_VARLEN", -1);
     opt.split_k = env_int("CUBERT_SPLIT_K", 1) != 0;
     opt.fuse_residual = env_int("CUBERT_FUSE_RESIDUAL", 1) != 0;
+    opt.fuse_layernorm = env_int("CUBERT_FUSE_LAYERNORM", 1) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;
@@ -292,6 +293,22 @@ int cubert_op_gemm_residual(const void* X, const void* W, const float* bias, con
     p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.elt = elt;
     p.out_elt = cubert::kF32; p.epilogue = cubert::kEpiBias; p.tile = tile; p.residual = R;
     apply_gemm_flags(&p, flags);
+    return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
+}
+
+size_t cubert_gemm_layernorm_workspace_bytes(int M) { return M > 0 ? cubert::gemm_ln_workspace_bytes((size_t)M) : 0; }
+
+int cubert_op_gemm_residual_layernorm(const void* X, const void* W, const float* bias, const float* R, const float* gamma,
+                                      const float* beta, float* Y, void* xb, void* workspace, int M, int N, int K, int ldx,
+                                      int tile, int flags, void* stream) {
+    cubert::set_error("");
+    if (!R || !gamma || !beta || !workspace) { cubert::set_error("cubert_op_gemm_residual_layernorm: null argument"); return 1; }
+    cubert::GemmParams p;
+    p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.elt = cubert::kBF16;
+    p.out_elt = cubert::kF32; p.epilogue = cubert::kEpiBias; p.tile = tile; p.residual = R;
+    p.ln_gamma = gamma; p.ln_beta = beta; p.ln_xb = xb; p.ln_xb_packed = (flags & CUBERT_Y_PACKED) != 0; p.ln_ws = workspace;
+    apply_gemm_flags(&p, flags);
+    p.y_packed = false;                 // CUBERT_Y_PACKED describes the bf16 copy here; Y itself is float32 row-major
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
 

@@ -56,6 +56,42 @@ __host__ __device__ inline size_t packed_offset(int r, int kbyte, int KB) {
            (kbyte & 15);
 }
 
+// ---- LayerNorm statistics -------------------------------------------------
+// Every LayerNorm of the engine (the row kernels and the GEMM epilogue that normalises) forms its
+// row statistics the same way, so that a row gets the same bits whichever kernel handles it:
+// the row is cut into slots of 128 features; in a slot 32 lanes hold four consecutive features each,
+// add them as (a + b) + (c + d) (squares likewise) and combine with ln_half_wave_sum; the slot sums are
+// added in slot order starting from zero; ln_finalize turns the totals into mean and 1 / sigma
+// (biased variance as E[x^2] - mean^2, eps 1e-12 inside the square root: cuda_bert/ops/layernorm.cu:
+// 127,167; modeling.py:168-172).
+#if defined(__HIPCC__)
+template <int CTRL>
+__device__ __forceinline__ float ln_dpp_lanes(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// Sum over the 32 lanes that share lane / 32; every lane gets the same bits (the additions are
+// pairwise and commutative).
+__device__ __forceinline__ float ln_half_wave_sum(float v) {
+    v += ln_dpp_lanes<0xB1>(v);       // quad_perm [1,0,3,2]: lane ^ 1
+    v += ln_dpp_lanes<0x4E>(v);       // quad_perm [2,3,0,1]: lane ^ 2
+    v += ln_dpp_lanes<0x141>(v);      // row_half_mirror: the other quad of 8 lanes
+    v += ln_dpp_lanes<0x140>(v);      // row_mirror: the other 8 of 16 lanes
+    v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));   // lane ^ 16
+    return v;
+}
+__device__ __forceinline__ float ln_sum4(float a, float b, float c, float d) { return (a + b) + (c + d); }
+__device__ __forceinline__ float ln_sumsq4(float a, float b, float c, float d) { return (a * a + b * b) + (c * c + d * d); }
+__device__ __forceinline__ void ln_finalize(float sum, float sumsq, float inv_n, float* mean, float* rstd) {
+    const float m = sum * inv_n;
+    const float var = fmaxf(sumsq * inv_n - m * m, 0.0f);
+    *mean = m;
+    *rstd = 1.0f / sqrtf(var + 1e-12f);
+}
+__device__ __forceinline__ float ln_apply(float x, float mean, float rstd, float gamma, float beta) {
+    return gamma * ((x - mean) * rstd) + beta;
+}
+#endif
+
 // Thread-local last error text (returned by cubert_last_error()).
 void set_error(const std::string& msg);
 const char* get_error();

@@ -196,6 +196,8 @@ bool Model::init(const ModelOptions& opt_in) {
     const size_t o_in = aa.take(3 * N * 4);
     const size_t meta_ints = N + (size_t)kMaxParts * kCuStride;
     const size_t o_meta = aa.take(meta_ints * 4), o_seqpad = aa.take(N * H * 4);
+    ln_ws_bytes_ = (gemm_ln_workspace_bytes(N) + 255) / 256 * 256;
+    const size_t o_lnws = aa.take(ln_ws_bytes_ * kMaxParts);
     act_bytes_ = aa.off;
     size_t free_b = 0, total_b = 0;
     CUBERT_HIP_OK(hipMemGetInfo(&free_b, &total_b));
@@ -218,6 +220,7 @@ bool Model::init(const ModelOptions& opt_in) {
     d_in_ = reinterpret_cast<int*>(ablock_ + o_in);
     d_meta_ = reinterpret_cast<int*>(ablock_ + o_meta);
     seqpad_ = reinterpret_cast<float*>(ablock_ + o_seqpad);
+    ln_ws_ = ablock_ + o_lnws;       // all zero from the clearing above, which is what the first launch needs
     CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_meta_), meta_ints * 4, hipHostMallocDefault));
     CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_in_), 3 * N * 4, hipHostMallocDefault));
     CUBERT_HIP_OK(hipStreamSynchronize(stream_));
@@ -347,13 +350,13 @@ bool Model::run_compact(const int* lens, int B, int S) {
     const size_t cu_off = cap + 256 * (kMaxParts - 1);
     CUBERT_HIP_OK(hipMemcpyAsync(d_meta_ + cu_off, h_meta_ + cu_off, (size_t)parts * kCuStride * 4, hipMemcpyHostToDevice, stream_));
     cur_parts_ = parts;
-    if (parts == 1) return enqueue_part(0, B, 0, S, false, stream_, &cp[0]);
+    if (parts == 1) return enqueue_part(0, 0, B, 0, S, false, stream_, &cp[0]);
     CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
     bool ok = true;
     for (int i = 0; i < parts; ++i) {
         hipStream_t st = i == 0 ? stream_ : side_[i];
         if (i > 0) CUBERT_HIP_OK(hipStreamWaitEvent(st, ev_fork_, 0));
-        ok = ok && enqueue_part(b0s[i], Bs[i], r0[i], S, false, st, &cp[i]);
+        ok = ok && enqueue_part(i, b0s[i], Bs[i], r0[i], S, false, st, &cp[i]);
         if (i > 0) {
             CUBERT_HIP_OK(hipEventRecord(ev_join_[i], st));
             CUBERT_HIP_OK(hipStreamWaitEvent(stream_, ev_join_[i], 0));
@@ -451,7 +454,7 @@ bool Model::enqueue(int B, int S, bool has_mask) {
     if (parts > B) parts = B;
     if (profiling_ || parts < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens) {
         cur_parts_ = 1;
-        return enqueue_part(0, B, 0, S, has_mask, stream_);
+        return enqueue_part(0, 0, B, 0, S, has_mask, stream_);
     }
     cur_parts_ = parts;
     CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
@@ -461,7 +464,7 @@ bool Model::enqueue(int B, int S, bool has_mask) {
         const int Bi = B / parts + (i < B % parts ? 1 : 0);
         hipStream_t st = i == 0 ? stream_ : side_[i];
         if (i > 0) CUBERT_HIP_OK(hipStreamWaitEvent(st, ev_fork_, 0));
-        ok = ok && enqueue_part(b0, Bi, r0, S, has_mask, st);
+        ok = ok && enqueue_part(i, b0, Bi, r0, S, has_mask, st);
         // join even after a failed launch so that a capture in progress can be closed
         if (i > 0) {
             CUBERT_HIP_OK(hipEventRecord(ev_join_[i], st));
@@ -478,7 +481,7 @@ bool Model::enqueue(int B, int S, bool has_mask) {
 // this part in the internal activation buffers (a multiple of 256, so that a
 // packed operand starts on a block boundary); inputs and the sequence output
 // are indexed by token.
-bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp) {
+bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp) {
     const Dims& D = opt_.dims;
     const int elt = opt_.precision;
     const size_t es = elt == kBF16 ? 2 : 4;
@@ -511,6 +514,12 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
     const int sp_ao = splits_for(H), sp_fo = splits_for(I);
     // the attn-out / FFN-out GEMMs add the residual stream in their epilogue, so LayerNorm reads one operand
     const bool fuse_res = opt_.fuse_residual;
+    // ... and, where the GEMM kernel can, normalise there as well: x32 and its bf16 copy come straight out of
+    // the GEMM and the LayerNorm launch disappears.  (Not with split K, whose parts the LayerNorm kernel adds.)
+    const bool ln_ao = fuse_res && opt_.fuse_layernorm && sp_ao == 1 && gemm_ln_supported(N, H, H, elt);
+    const bool ln_fo = fuse_res && opt_.fuse_layernorm && sp_fo == 1 && gemm_ln_supported(N, H, I, elt);
+    void* ln_ws = ln_ws_ + (size_t)part * ln_ws_bytes_;
+    if (ln_ao || ln_fo) ln_used_ = true;
 
     if (!mark(kPhEmbed)) return false;
     const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
@@ -534,9 +543,10 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;
         g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_ao;
         g.residual = fuse_res ? x32 : nullptr;
+        if (ln_ao) { g.Y = x32; g.ln_gamma = L.g1; g.ln_beta = L.be1; g.ln_xb = xb; g.ln_xb_packed = pk; g.ln_ws = ln_ws; }
         if (!mark(kPhAttnOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st, sp_ao, !fuse_res)) return false;
+        if (!ln_ao && !launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st, sp_ao, !fuse_res)) return false;
         // feed-forward
         g = GemmParams();
         g.elt = elt; g.out_elt = elt; g.X = xin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = h;
@@ -546,9 +556,10 @@ bool Model::enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStre
         g.elt = elt; g.out_elt = kF32; g.X = h; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32;
         g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_fo;
         g.residual = fuse_res ? x32 : nullptr;
+        if (ln_fo) { g.Y = x32; g.ln_gamma = L.g2; g.ln_beta = L.be2; g.ln_xb = xb; g.ln_xb_packed = pk; g.ln_ws = ln_ws; }
         if (!mark(kPhFFNOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
-        if (!launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st, sp_fo, !fuse_res)) return false;
+        if (!ln_fo && !launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st, sp_fo, !fuse_res)) return false;
     }
     // pooler: first-token gather + dense + tanh on the float32 sequence output
     if (!mark(kPhPooler)) return false;
@@ -588,7 +599,7 @@ bool Model::profile_device(const int* d_ids, const int* d_seg, const int* d_mask
     ok = ok && mark(-1);                       // closing event
     profiling_ = false;
     if (!ok) return false;
-    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    if (!sync()) return false;
     for (int i = 0; i < kNumPhases; ++i) phase_ms[i] = 0.0f;
     for (size_t i = 0; i + 1 < prof_used_; ++i) {
         float ms = 0.0f;
@@ -606,6 +617,20 @@ bool Model::classify() {
 
 bool Model::sync() {
     CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    if (ln_used_) {
+        // A workgroup of a GEMM that normalises in its epilogue gives up after a bounded wait for its
+        // partners and raises word 0 of its workspace; the results of that pass are then not valid.
+        ln_used_ = false;
+        for (int i = 0; i < kMaxParts; ++i) {
+            int flag = 0;
+            CUBERT_HIP_OK(hipMemcpy(&flag, ln_ws_ + (size_t)i * ln_ws_bytes_, sizeof(int), hipMemcpyDeviceToHost));
+            if (flag != 0) {
+                CUBERT_HIP_OK(hipMemset(ln_ws_ + (size_t)i * ln_ws_bytes_, 0, ln_ws_bytes_));
+                set_error("a GEMM with the LayerNorm in its epilogue timed out waiting for the workgroups it shares rows with");
+                return false;
+            }
+        }
+    }
     return true;
 }
 

@@ -27,6 +27,7 @@ struct ModelOptions {
     int split_parts = 2;           // number of parts (1..4) a large batch is cut into
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
     bool fuse_residual = true;     // residual add in the epilogue of the GEMM before each LayerNorm
+    bool fuse_layernorm = true;    // ... and the LayerNorm itself, where the GEMM kernel supports it (bf16, large batches)
     bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
     int varlen = -1;               // host-input calls with prefix masks compute only the valid tokens: 1 always,
                                    // 0 never, -1 when the caller asks for no sequence output (see forward_host)
@@ -88,7 +89,7 @@ class Model {
     bool check_shape(int B, int S);
     bool run(int B, int S, bool has_mask);             // graph or eager
     bool enqueue(int B, int S, bool has_mask);         // the launch sequence (one or two parts)
-    bool enqueue_part(int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp = nullptr);
+    bool enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp = nullptr);
     bool run_compact(const int* h_lens, int B, int S);
     bool mark(int phase);                              // profiling: event before a launch
 
@@ -125,6 +126,9 @@ class Model {
     int* d_meta_ = nullptr;      // rowmap (cap tokens) | cu (kMaxParts * kCuStride)
     int* h_meta_ = nullptr;      // pinned, same layout
     float* seqpad_ = nullptr;    // padded [B, S, H] sequence output of an unpadded pass
+    unsigned char* ln_ws_ = nullptr;   // kMaxParts workspaces of the GEMMs that normalise in their epilogue
+    size_t ln_ws_bytes_ = 0;           // size of one of them
+    bool ln_used_ = false;             // such a GEMM ran since sync() last looked at the workspaces' error words
     bool last_compact_ = false;
     int cur_parts_ = 1;          // parts of the pass being enqueued
     int B_ = 0, S_ = 0;

@@ -38,6 +38,7 @@ namespace cubert {
 
 bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
 bool launch_gemm_bf16_t256x128(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
+int gemm_pick_tile(int M, int N, int K, int elt);
 
 namespace {
 
@@ -275,6 +276,26 @@ bool launch_epi(const GemmDev& d, int epi, int bt, hipStream_t stream) {
 
 }  // namespace
 
+namespace {
+// Workspace of the LayerNorm epilogue: flag words, two counters per band of rows (a fixed number of
+// bands, so that launches with different M agree on where the counters are), then (sum, sum of squares)
+// for every row and every 128-feature slot (at most 8).
+constexpr size_t kLnMaxBands = 16384;
+size_t ln_stats_offset() { return ((gemm_detail::kLnCntFirst + 2 * kLnMaxBands) * sizeof(int) + 255) / 256 * 256; }
+}  // namespace
+
+size_t gemm_ln_workspace_bytes(size_t M) { return ln_stats_offset() + ((M + 255) / 256 * 256) * 8 * sizeof(unsigned long long); }
+
+namespace {
+bool ln_shape_ok(int N, int K, int elt) { return elt == kBF16 && N > 0 && N % 256 == 0 && N <= 1024 && K % 32 == 0 && K >= 64; }
+}  // namespace
+
+bool gemm_ln_supported(int M, int N, int K, int elt) {
+    if (M <= 0 || !ln_shape_ok(N, K, elt)) return false;
+    const int bt = gemm_pick_tile(M, N, K, elt);
+    return bt == kTile256x128 || (bt == 256 && K % 128 == 0);
+}
+
 int gemm_pick_tile(int M, int N, int K, int elt) {
     auto tiles = [&](int bt) { return (long)((M + bt - 1) / bt) * ((N + bt - 1) / bt); };
     auto rounds = [](long wgs, long slots) { return (double)((wgs + slots - 1) / slots); };
@@ -336,7 +357,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     d.x_packed = p.x_packed; d.w_packed = p.w_packed; d.y_packed = p.y_packed;
     int out = p.out_elt;
     int epi = (p.epilogue == kEpiQKV && p.rowmap) ? (int)kEpiQKVMap : p.epilogue;
-    if (p.epilogue == kEpiQKVMap || p.epilogue == kEpiBiasRes) { set_error("gemm: unknown epilogue"); return false; }
+    if (p.epilogue == kEpiQKVMap || p.epilogue == kEpiBiasRes || p.epilogue == kEpiBiasResLN) { set_error("gemm: unknown epilogue"); return false; }
     if (p.residual) {
         if (p.epilogue != kEpiBias || out != kF32 || p.y_packed || p.N % 4 != 0 ||
             (reinterpret_cast<uintptr_t>(p.residual) & 15)) {
@@ -345,6 +366,26 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         }
         epi = kEpiBiasRes;
         d.R = p.residual;
+    }
+    if (p.ln_gamma) {
+        if (!p.residual || !p.ln_beta || !p.ln_ws || p.splits > 1 || !ln_shape_ok(p.N, p.K, p.elt) ||
+            ((size_t)p.M + 256) * p.N * 4 >= (1ull << 31) || (size_t)(p.M + 127) / 128 > kLnMaxBands ||
+            (p.tile ? (p.tile != 256 && p.tile != kTile256x128) || (p.tile == 256 && p.K % 128 != 0)
+                    : !gemm_ln_supported(p.M, p.N, p.K, p.elt)) ||
+            ((reinterpret_cast<uintptr_t>(p.ln_gamma) | reinterpret_cast<uintptr_t>(p.ln_beta) |
+              reinterpret_cast<uintptr_t>(p.ln_xb) | reinterpret_cast<uintptr_t>(p.ln_ws)) & 15)) {
+            set_error("gemm: the LayerNorm epilogue needs a residual, bf16 operands, N a multiple of 256 up to 1024, the "
+                      "256 or 256x128 tile, no split K, a workspace and 16-byte aligned gamma / beta / copy");
+            return false;
+        }
+        epi = kEpiBiasResLN;
+        d.ln_gamma = p.ln_gamma;
+        d.ln_beta = p.ln_beta;
+        d.ln_xb = static_cast<unsigned char*>(p.ln_xb);
+        d.ln_xb_packed = p.ln_xb_packed ? 1 : 0;
+        d.ln_bands = (int)kLnMaxBands;
+        d.ln_cnt = static_cast<int*>(p.ln_ws);
+        d.ln_stats = reinterpret_cast<unsigned long long*>(static_cast<unsigned char*>(p.ln_ws) + ln_stats_offset());
     }
     if (p.epilogue == kEpiQKV) {
         if (!p.q || !p.k || !p.vt || p.S <= 0 || p.heads <= 0 || p.N != 3 * p.heads * 64 ||
@@ -375,7 +416,11 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         }
     }
     int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
+    // With the LayerNorm in the epilogue the 256 x 256 tile measured faster than 256 x 128 wherever both apply
+    // (one exchange per 256 rows instead of two, and the long epilogue does not share the CU's LDS pipe).
+    if (epi == kEpiBiasResLN && !p.tile && p.K % 128 == 0) bt = 256;
     if (d.splits > 1 && bt == 256 && !p.tile) bt = 128;      // the hand-scheduled kernel does not split
+    if (epi == kEpiBiasResLN && p.compiler_scheduled) { set_error("gemm: the LayerNorm epilogue has no compiler-scheduled kernel"); return false; }
     if (bt == kTile256x128) {
         if (p.elt != kBF16 || d.splits != 1) { set_error("gemm: the 256x128 tile is bf16 only and does not split K"); return false; }
         d.tiles_n = (p.N + 255) / 256;

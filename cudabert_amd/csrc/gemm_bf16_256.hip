@@ -35,7 +35,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
     const int l32 = lane & 31, g = lane >> 5;
 
     int tile_n, tile_m;
-    tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
+    if constexpr (EPI == kEpiBiasResLN) {
+        ln_tile_of_block(blockIdx.x, p.tiles_n, &tile_n, &tile_m);
+        if (tile_m >= p.tiles_m) return;          // the grid is padded to whole groups of eight bands
+    } else {
+        tile_of_block(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
+    }
     const int n0 = tile_n * BT, m0 = tile_m * BT;
 
     // Buffer descriptors as plain SGPR quads: base, base_hi (stride 0), num_records, flags.
@@ -85,7 +90,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_t256_kernel(const GemmDev p) {
 
     // Stages 0 and 1 were last read two barriers ago; the tail of the loop only reads stages
     // 2 and 3, so the first 64 KiB are free for the epilogue's staging while slower waves finish.
-    gemm_epilogue<OUT, EPI, 4, 4, false, 8, true>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
+    // (The LayerNorm epilogue keeps its row statistics above them, after a barrier of its own.)
+    if constexpr (EPI == kEpiBiasResLN)
+        gemm_epilogue_ln<4, 4>(p, acc, n0 + wn * 128, m0 + wm * 128, l32, g, tile_m, 2 * tile_n + wn, lds + wave * 16384,
+                               reinterpret_cast<float*>(lds + 65536 + wave * 1024));
+    else
+        gemm_epilogue<OUT, EPI, 4, 4, false, 8, true>(p, acc, bias, n0 + wn * 128, m0 + wm * 128, l32, g, lds + wave * 16384);
 }
 
 // ---------------------------------------------------------------------------
@@ -110,7 +120,12 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
     const int l32 = lane & 31, g = lane >> 5;
 
     int tile_n, tile_m;
-    tile_of_block<8>(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
+    if constexpr (EPI == kEpiBiasResLN) {
+        ln_tile_of_block(blockIdx.x, p.tiles_n, &tile_n, &tile_m);
+        if (tile_m >= p.tiles_m) return;          // the grid is padded to whole groups of eight bands
+    } else {
+        tile_of_block<8>(blockIdx.x, p.tiles_n * p.tiles_m, p.tiles_n, p.xn_parts, &tile_n, &tile_m);
+    }
     const int n0 = tile_n * 256, m0 = tile_m * 128;
 
     const unsigned long long wa = reinterpret_cast<unsigned long long>(p.W);
@@ -152,8 +167,16 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
     // The block ends with all loads landed and a barrier: the whole LDS is free for staging.
     f32x4_t bias[16];
     if constexpr (!gemm_bias_at_readout<OUT, EPI>()) gemm_load_bias<4>(p, n0 + wn * 128, g, bias);
-    gemm_epilogue<OUT, EPI, 4, 2, false, 8, true>(p, acc, bias, n0 + wn * 128, m0 + wm * 64, l32, g, lds + wave * 16384);
+    if constexpr (EPI == kEpiBiasResLN)
+        gemm_epilogue_ln<4, 2>(p, acc, n0 + wn * 128, m0 + wm * 64, l32, g, tile_m, 2 * tile_n + wn, lds + wave * 16384,
+                               reinterpret_cast<float*>(lds + 65536 + wave * 1024));
+    else
+        gemm_epilogue<OUT, EPI, 4, 2, false, 8, true>(p, acc, bias, n0 + wn * 128, m0 + wm * 64, l32, g, lds + wave * 16384);
 }
+
+// LayerNorm epilogue: eight XCDs x whole groups of bands x the workgroups of a band (ln_tile_of_block);
+// workgroups whose band does not exist leave at once.
+dim3 ln_grid(const GemmDev& d) { return dim3(8 * d.tiles_n * ((d.tiles_m + 7) / 8)); }
 
 template <int OUT>
 bool launch_epi_half(const GemmDev& d, int epi, hipStream_t stream) {
@@ -168,6 +191,14 @@ bool launch_epi_half(const GemmDev& d, int epi, hipStream_t stream) {
             if constexpr (OUT == kF32) {
                 hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBiasRes>), grid, block, 0, stream, d);
                 break;
+            }
+            [[fallthrough]];
+        case kEpiBiasResLN:
+            if constexpr (OUT == kF32) {
+                if (epi == kEpiBiasResLN) {
+                    hipLaunchKernelGGL((gemm_bf16_t256x128_kernel<OUT, kEpiBiasResLN>), ln_grid(d), block, 0, stream, d);
+                    break;
+                }
             }
             [[fallthrough]];
         default: set_error("gemm: unknown epilogue"); return false;
@@ -189,6 +220,14 @@ bool launch_epi(const GemmDev& d, int epi, hipStream_t stream) {
             if constexpr (OUT == kF32) {
                 hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasRes>), grid, block, 0, stream, d);
                 break;
+            }
+            [[fallthrough]];
+        case kEpiBiasResLN:
+            if constexpr (OUT == kF32) {
+                if (epi == kEpiBiasResLN) {
+                    hipLaunchKernelGGL((gemm_bf16_t256_kernel<OUT, kEpiBiasResLN>), ln_grid(d), block, 0, stream, d);
+                    break;
+                }
             }
             [[fallthrough]];
         default: set_error("gemm: unknown epilogue"); return false;

@@ -11,6 +11,7 @@ typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2_t;
 
 struct GemmDev {
     const unsigned char* X;
@@ -28,7 +29,18 @@ struct GemmDev {
     const int* rowmap;                    // QKV epilogue: row m -> token b * S + s (nullptr: m itself)
     const float* R;                       // kEpiBiasRes: [M, N] float32 row-major, added to the result
     int splits;                           // split K: blockIdx.y owns a K range, results go to Y + y * M * N (f32)
+    // kEpiBiasResLN: LayerNorm in the epilogue (gemm_epilogue_ln)
+    const float* ln_gamma;
+    const float* ln_beta;
+    unsigned char* ln_xb;                 // bf16 copy of the result (may be null)
+    int ln_xb_packed;
+    int* ln_cnt;                          // [0] error flag, [kLnCntFirst + band] arrivals, [.. + ln_bands + band] departures
+    unsigned long long* ln_stats;         // [row][2 * tiles_n] (sum, sum of squares) as two floats in 64 bits
+    int ln_bands;
 };
+
+constexpr int kLnCntFirst = 64;           // first counter word of the workspace (the words before it: flags)
+constexpr int kLnSpinLimit = 1 << 21;     // polls of a band's arrival counter before a workgroup gives up
 
 __device__ __forceinline__ float gelu_erf(float x) {
     return x * 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
@@ -155,7 +167,7 @@ inline int gemm_pick_partition(double x_bytes, double w_bytes, int tiles_n, int 
 // a lane serves one group of four features for all rows (one quad instead of 4 NB): gemm_load_bias is
 // not needed for them and the epilogue ignores its `bias` argument.
 template <int OUT, int EPI>
-constexpr bool gemm_bias_at_readout() { return OUT == kF32 && (EPI == kEpiBias || EPI == kEpiBiasRes); }
+constexpr bool gemm_bias_at_readout() { return OUT == kF32 && (EPI == kEpiBias || EPI == kEpiBiasRes || EPI == kEpiBiasResLN); }
 
 // The bias values a lane needs (4 NB quads) are fetched by gemm_load_bias before the
 // K loop so that their latency is hidden; features past N read the last valid quad
@@ -309,6 +321,233 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             } else {
                 const size_t part = SPLITK ? (size_t)blockIdx.y * p.M : 0;
                 *reinterpret_cast<u32x4_t*>(p.Y + ((part + mm) * p.N + n) * OES) = d;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm in the epilogue (kEpiBiasResLN): Y = LayerNorm(acc + bias + R) * gamma + beta over rows of
+// N = 256 * tiles_n features, float32 row-major, plus an optional bf16 copy (the next GEMM's operand).
+//
+// A workgroup holds 256 of a row's features, so the tiles_n workgroups of one band of rows have to
+// agree on the row statistics.  Every wave (128 features of its rows) publishes (sum, sum of squares)
+// per row in device memory, the workgroup counts itself in on the band's arrival counter, waits until
+// all tiles_n workgroups have, and reads the 2 * tiles_n partial sums of its rows.  The accumulators go
+// through the wave's LDS staging once (whole row segments come out, bias and residual are added to
+// them); the sums go back into the registers the accumulators came from and wait there, in read-out
+// order, until the statistics are known, and are then normalised and stored.
+//
+// Workgroup order (ln_tile_of_block): XCD x (= workgroup id % 8) owns the bands x, x + 8, ...; the
+// workgroups of a band have consecutive positions on that XCD, i.e. ids 8 apart.  Workgroups are
+// dispatched in id order per XCD, so whenever 32 workgroups of the launch are resident the partners of
+// the oldest unfinished one are resident or done, and it can finish: no deadlock however many CUs
+// other launches occupy (two such launches cannot both hold fewer than 32 of the 256 CUs for ever).
+// The wait is bounded all the same (kLnSpinLimit polls); a workgroup that gives up raises the error
+// word of the workspace and stores what it has.
+//
+// The counters of a band are put back to zero by the last workgroup to leave it, so the workspace
+// needs no clearing between launches (and none inside a captured graph).
+__device__ __forceinline__ void ln_tile_of_block(int pid, int tiles_n, int* tn, int* tm) {
+    const int xcd = pid & 7, idx = pid >> 3;
+    *tm = (idx / tiles_n) * 8 + xcd;
+    *tn = idx % tiles_n;
+}
+
+// One trip of the accumulators through the wave's LDS staging block: block column j is written in
+// accumulator order (row = token, chunk swizzled by the row) and read back as whole row segments, lane
+// (rrow, rc) taking features 4 rc .. 4 rc + 3 of row 2 s + rrow in step s; bias and residual are added on
+// the way out and `use(j, s, d)` receives the sums.  The residual rows come in batches of PB steps, the
+// next batch requested before the current one is consumed.
+template <int NBI, int NBJ, int SCHED, typename Use>
+__device__ __forceinline__ void ln_stream_rows(f32x16_t (&acc)[NBI][NBJ], unsigned char* buf, int l32, int g, int rrow, int rc,
+                                               const f32x4_t& bias4, __amdgpu_buffer_rsrc_t r_rsrc, int lane_off, int row_bytes,
+                                               Use use) {
+    constexpr int RB = 512, RPI = 2, NIT = 16, PB = 8;
+    constexpr int NBATCH = NBJ * NIT / PB;
+    f32x4_t res[2][PB];
+    auto fetch_res = [&](int batch, f32x4_t (&r)[PB]) {
+#pragma unroll
+        for (int u = 0; u < PB; ++u)      // row 32 j + 2 s (+ rrow) with j * NIT + s = batch * PB + u
+            r[u] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(r_rsrc, lane_off + (batch * PB + u) * RPI * row_bytes, 0, 0));
+    };
+    fetch_res(0, res[0]);
+#pragma unroll
+    for (int j = 0; j < NBJ; ++j) {
+#pragma unroll
+        for (int i = 0; i < NBI; ++i)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int fb = (32 * i + 8 * qd + 4 * g) * 4;
+                const f32x4_t v = {acc[i][j][4 * qd], acc[i][j][4 * qd + 1], acc[i][j][4 * qd + 2], acc[i][j][4 * qd + 3]};
+                *reinterpret_cast<f32x4_t*>(buf + l32 * RB + ((((fb >> 4) ^ l32) & 31) << 4)) = v;
+            }
+#pragma unroll
+        for (int s = 0; s < NIT; ++s) {
+            const int batch = (j * NIT + s) / PB;             // compile-time after unrolling
+            if (s % PB == 0 && batch + 1 < NBATCH) fetch_res(batch + 1, res[(batch + 1) & 1]);
+            const int row = s * RPI + rrow;
+            const f32x4_t staged = *reinterpret_cast<const f32x4_t*>(buf + row * RB + (((rc ^ row) & 31) << 4));
+            use(j, s, (staged + bias4) + res[batch & 1][s % PB]);
+            if (s % SCHED == SCHED - 1) __builtin_amdgcn_sched_barrier(0);     // bounds how many steps the scheduler interleaves
+        }
+    }
+}
+
+template <int NBI, int NBJ>
+__device__ __forceinline__ void gemm_epilogue_ln(const GemmDev& p, f32x16_t (&acc)[NBI][NBJ], int n_base, int m_base,
+                                                 int l32, int g, int band, int slot, unsigned char* buf,
+                                                 float* statbuf) {
+    static_assert(NBI == 4 && NBJ % 2 == 0, "a wave holds 128 features and a multiple of 64 rows");
+    constexpr int RPI = 2;                   // rows one read-out step covers
+    constexpr int NIT = 16;                  // read-out steps per block column of 32 rows
+    constexpr int NP = NBJ * NIT / 32;       // (block column, step) pairs whose row a lane publishes
+    const int slots = 2 * p.tiles_n;
+    const float invn = 1.0f / (float)p.N;
+    // Residual and result through buffer descriptors: a row's address is one lane offset plus a
+    // wave-uniform row term, rows past M read as zero and are not stored.  (The whole offset goes
+    // into the lane operand: the descriptor's range check does not look at the scalar offset.)
+    const int row_bytes = p.N * 4;
+    const __amdgpu_buffer_rsrc_t r_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.R), 0, p.M * row_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t y_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.Y, 0, p.M * row_bytes, 0x00020000);
+
+    // ---- first pass: row sums of (acc + bias + R) over this wave's 128 features ----
+    float ksum[NP], ksq[NP];
+#pragma unroll
+    for (int t = 0; t < NP; ++t) ksum[t] = ksq[t] = 0.0f;
+    {
+        const int lane = l32 + 32 * g, rrow = lane >> 5, rc = lane & 31;
+        const int n = n_base + rc * 4;           // this lane's four features on the way out (N % 256 == 0: in range)
+        const f32x4_t bias4 = *reinterpret_cast<const f32x4_t*>(p.bias + n);
+        ln_stream_rows<NBI, NBJ, 4>(acc, buf, l32, g, rrow, rc, bias4, r_rsrc, (m_base + rrow) * row_bytes + n * 4, row_bytes,
+                                 [&](int j, int s, const f32x4_t& d) {
+            const float t = ln_half_wave_sum(ln_sum4(d[0], d[1], d[2], d[3]));
+            const float q = ln_half_wave_sum(ln_sumsq4(d[0], d[1], d[2], d[3]));
+            const int pair = j * NIT + s;                     // compile-time after unrolling
+            if (rc == (pair & 31)) { ksum[pair >> 5] = t; ksq[pair >> 5] = q; }
+            // The sums stay in the registers of the accumulators they were made from (block column j
+            // has been staged completely by now): step s of column j in acc[s / 4][j][4 (s % 4) ..].
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[s / 4][j][4 * (s % 4) + e] = d[e];
+            // the selection happens here (left to itself the compiler postpones all of them past the
+            // loop and spills every step's sums until then)
+            asm volatile("" : "+v"(ksum[pair >> 5]), "+v"(ksq[pair >> 5]));
+        });
+        // lane (rrow, rc) publishes the rows of the pairs t * 32 + rc
+#pragma unroll
+        for (int t = 0; t < NP; ++t) {
+            const int pair = t * 32 + rc;
+            const int mm = m_base + 32 * (pair / NIT) + RPI * (pair % NIT) + rrow;
+            if (mm < p.M) {
+                const unsigned long long bits = (unsigned long long)__builtin_bit_cast(unsigned, ksum[t]) |
+                                                ((unsigned long long)__builtin_bit_cast(unsigned, ksq[t]) << 32);
+                __hip_atomic_store(p.ln_stats + (size_t)mm * slots + slot, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the sums are in place before the workgroup counts itself in
+    __syncthreads();
+    int* arrivals = p.ln_cnt + kLnCntFirst + band;
+    int* departures = arrivals + p.ln_bands;
+    if (threadIdx.x == 0) {
+        __hip_atomic_fetch_add(arrivals, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int polls = 0;
+        while (__hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p.tiles_n) {
+            if (++polls > kLnSpinLimit) {
+                __hip_atomic_store(p.ln_cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+    }
+    __syncthreads();
+
+    // What the registers of the accumulators hold now (the sums, in read-out order) has to survive
+    // the wait in place: the empty statements keep the compiler from moving the values elsewhere.
+#pragma unroll
+    for (int i = 0; i < NBI; ++i)
+#pragma unroll
+        for (int j = 0; j < NBJ; ++j) asm volatile("" : "+a"(acc[i][j]));
+    // (Likewise the lane coordinates: from laundered copies, so that the addresses of the second pass
+    // are formed after the wait instead of being carried, and spilled, through the first.)
+    int l32b = l32, gb = g;
+    asm volatile("" : "+v"(l32b), "+v"(gb));
+    const int lane = l32b + 32 * gb, rrow = lane >> 5, rc = lane & 31;
+    const int n = n_base + rc * 4;
+
+    // ---- statistics of my rows: all partial sums, in slot order ----
+    // The partners' sums are read with cache-bypassing buffer loads (sc0 | sc1), all requested before the
+    // first one is used.  A row's slots are contiguous: a load past 2 * tiles_n reads the next row's or,
+    // at the end, nothing (zero); those values are not added.
+    {
+        const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.ln_stats, 0, p.M * slots * 8, 0x00020000);
+        f32x4_t raw[NP][4];
+#pragma unroll
+        for (int t = 0; t < NP; ++t) {
+            const int pair = t * 32 + rc;
+            const int mm = m_base + 32 * (pair / NIT) + RPI * (pair % NIT) + rrow;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)          // two slots per load; rows past M fall outside the descriptor as well
+                raw[t][c] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(s_rsrc, (mm * slots + 2 * c) * 8, 0, 17));
+        }
+#pragma unroll
+        for (int t = 0; t < NP; ++t) {
+            const int pair = t * 32 + rc;
+            const int rl = 32 * (pair / NIT) + RPI * (pair % NIT) + rrow;     // row within the wave's rows
+            float sum = 0.0f, sq = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (2 * c < slots) {          // a wave-uniform branch; slots is even
+                    sum += raw[t][c][0]; sq += raw[t][c][1];
+                    sum += raw[t][c][2]; sq += raw[t][c][3];
+                }
+            }
+            float mean, rstd;
+            ln_finalize(sum, sq, invn, &mean, &rstd);
+            statbuf[2 * rl] = mean;
+            statbuf[2 * rl + 1] = rstd;
+        }
+    }
+    __syncthreads();                                       // every wave holds its statistics: the band can be left
+    if (threadIdx.x == 0) {
+        if (__hip_atomic_fetch_add(departures, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.tiles_n - 1) {
+            __hip_atomic_store(arrivals, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(departures, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+
+    // ---- second pass: normalise the kept sums and store ----
+    const f32x4_t gamma4 = *reinterpret_cast<const f32x4_t*>(p.ln_gamma + n);
+    const f32x4_t beta4 = *reinterpret_cast<const f32x4_t*>(p.ln_beta + n);
+    // bf16 copy: row-major, or packed (common.h): block of 256 rows x 64 bytes, chunk c of row r in slot
+    // c ^ ((r >> 2) & 3).  The wave's rows start at a multiple of 64, so with r = m_base + 32 j + 2 s + rrow
+    // the row's block and its swizzle (s >> 1) & 3 are known per step; only the chunk is the lane's.
+    const bool xb_on = p.ln_xb != nullptr;
+    const int xb_size = p.ln_xb_packed ? (int)packed_bytes(p.M, (size_t)p.N * 2) : p.M * p.N * 2;
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(xb_on ? p.ln_xb : p.Y, 0, xb_on ? xb_size : 0, 0x00020000);
+    const int kb_per_row = p.N * 2 / 64;
+    const int xb_chunk = (n * 2 >> 4) & 3;
+    const int xb_lane = p.ln_xb_packed
+        ? (((m_base >> 8) * kb_per_row + (n * 2 >> 6)) * 16384 + ((m_base & 255) + rrow) * 64 + ((n * 2) & 15))
+        : ((m_base + rrow) * p.N + n) * 2;
+    const int lane_off = (m_base + rrow) * row_bytes + n * 4;
+#pragma unroll
+    for (int j = 0; j < NBJ; ++j) {
+#pragma unroll
+        for (int s = 0; s < NIT; ++s) {
+            const int step_rows = 32 * j + s * RPI;
+            const int rl = step_rows + rrow;
+            const float mean = statbuf[2 * rl], rstd = statbuf[2 * rl + 1];
+            f32x4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = ln_apply(acc[s / 4][j][4 * (s % 4) + e], mean, rstd, gamma4[e], beta4[e]);
+            // rows past M: the descriptor drops the float32 store; the copy is predicated
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, o), y_rsrc, lane_off + step_rows * row_bytes, 0, 0);
+            if (xb_on && m_base + rl < p.M) {
+                const bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
+                const int off = p.ln_xb_packed ? xb_lane + step_rows * 64 + ((xb_chunk ^ ((s >> 1) & 3)) << 4)
+                                               : xb_lane + step_rows * p.N * 2;
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2_t, ob), x_rsrc, off, 0, 0);
             }
         }
     }

@@ -24,6 +24,7 @@ enum GemmEpilogue : int {
     kEpiQKV = 3,       // scatter into per-head Q, K and transposed V (see below)
     kEpiQKVMap = 4,    // the same on compact rows: row m is token rowmap[m] (chosen by launch_gemm when rowmap is set)
     kEpiBiasRes = 5,   // Y = acc + bias + R, float32 row-major (chosen by launch_gemm when residual is set)
+    kEpiBiasResLN = 6, // Y = LayerNorm(acc + bias + R) (chosen by launch_gemm when ln_gamma is set)
 };
 
 // Unpadded ("compact") rows: only the valid tokens of every sequence are stored,
@@ -58,6 +59,19 @@ struct GemmParams {
     // kEpiBias with a float32 row-major Y: [M, N] float32 added to the result (the residual branch of
     // the layer, so that the LayerNorm after it reads one operand).  With split K it goes into partial 0.
     const float* residual = nullptr;
+    // kEpiBias with a residual and ln_gamma set: the LayerNorm that follows the linear runs in the
+    // epilogue.  Y (float32 row-major, may be the residual buffer itself) receives
+    // LayerNorm(acc + bias + R) * gamma + beta over each row of N features, ln_xb (optional) a bf16
+    // copy of it (row-major, or packed with ln_xb_packed).  bf16 operands, the 256 x 256 or 256 x 128
+    // tile, N a multiple of 256 up to 1024, no split K.  The N / 256 workgroups that hold one band
+    // of rows exchange their partial row sums through ln_ws: gemm_ln_workspace_bytes(M) bytes of
+    // device memory that are all zero before the first launch (each launch leaves the words it
+    // counts with at zero again), used by one launch at a time.
+    const float* ln_gamma = nullptr;
+    const float* ln_beta = nullptr;
+    void* ln_xb = nullptr;
+    bool ln_xb_packed = false;
+    void* ln_ws = nullptr;
     int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile) or kTile256x128
     // Split K (kEpiBias, float32 Y): `splits` workgroups share a tile, each reduces its share of K and
     // writes its partial result to Y + z * M * N; the bias goes into partial 0.  The consumer adds
@@ -68,6 +82,11 @@ struct GemmParams {
     bool x_packed = false, w_packed = false, y_packed = false;
 };
 bool launch_gemm(const GemmParams& p, hipStream_t stream);
+// Workspace of a GEMM with the LayerNorm in its epilogue (GemmParams::ln_ws) for up to M rows.
+size_t gemm_ln_workspace_bytes(size_t M);
+// True if launch_gemm can run the LayerNorm of a [M, N] float32 result in the epilogue of a
+// bf16 GEMM with reduction length K.
+bool gemm_ln_supported(int M, int N, int K, int elt);
 
 // ----------------------------------------------------------- attention -----
 // Fused QK^T * scale + mask -> softmax -> P V for head dim 64.

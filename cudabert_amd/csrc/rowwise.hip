@@ -32,23 +32,24 @@ __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H
                                                 const float* __restrict__ gamma,
                                                 const float* __restrict__ beta, float* xrow,
                                                 bf16_t* xb, int row, int xb_packed) {
-    float s = 0.0f;
+    // Row statistics in the engine's canonical order (common.h): chunk c holds the slots 2 c (lanes
+    // 0..31) and 2 c + 1 (lanes 32..63); slots past the row's end contribute zero.
+    float sum = 0.0f, sumsq = 0.0f;
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c)
-        if (c * 256 + lane * 4 < H) s += (v[c][0] + v[c][1]) + (v[c][2] + v[c][3]);
-    const float mean = wave_sum(s) / (float)H;
-    float sq = 0.0f;
-#pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c)
-        if (c * 256 + lane * 4 < H) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[c][e] -= mean;
-                sq += v[c][e] * v[c][e];
-            }
-        }
-    const float var = wave_sum(sq) / (float)H;
-    const float rstd = 1.0f / sqrtf(var + 1e-12f);
+    for (int c = 0; c < kMaxChunks; ++c) {
+        const bool in = c * 256 + lane * 4 < H;
+        const float t = ln_half_wave_sum(in ? ln_sum4(v[c][0], v[c][1], v[c][2], v[c][3]) : 0.0f);
+        const float q = ln_half_wave_sum(in ? ln_sumsq4(v[c][0], v[c][1], v[c][2], v[c][3]) : 0.0f);
+        // every lane gets the lower slot's sum first, then the upper one's
+        const float t_other = __shfl_xor(t, 32), q_other = __shfl_xor(q, 32);
+        const bool upper = lane >= 32;
+        sum += upper ? t_other : t;
+        sumsq += upper ? q_other : q;
+        sum += upper ? t : t_other;
+        sumsq += upper ? q : q_other;
+    }
+    float mean, rstd;
+    ln_finalize(sum, sumsq, 1.0f / (float)H, &mean, &rstd);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
         const int i = c * 256 + lane * 4;
@@ -57,7 +58,7 @@ __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H
             const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(beta + i);
             f32x4_t o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = g4[e] * (v[c][e] * rstd) + b4[e];
+            for (int e = 0; e < 4; ++e) o[e] = ln_apply(v[c][e], mean, rstd, g4[e], b4[e]);
             __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t*>(xrow + i));
             if (xb) {
                 bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};

@@ -106,6 +106,10 @@ lib.cubert_op_gemm.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_
 lib.cubert_op_gemm.restype = c_int
 lib.cubert_op_gemm_residual.argtypes = [c_void_p] * 5 + [c_int] * 7 + [c_void_p]
 lib.cubert_op_gemm_residual.restype = c_int
+lib.cubert_gemm_layernorm_workspace_bytes.argtypes = [c_int]
+lib.cubert_gemm_layernorm_workspace_bytes.restype = ctypes.c_size_t
+lib.cubert_op_gemm_residual_layernorm.argtypes = [c_void_p] * 9 + [c_int] * 6 + [c_void_p]
+lib.cubert_op_gemm_residual_layernorm.restype = c_int
 lib.cubert_op_gemm_splitk_noalloc.argtypes = [c_void_p] * 4 + [c_int] * 8 + [c_void_p]
 lib.cubert_op_gemm_splitk_noalloc.restype = c_int
 lib.cubert_noalloc_scratch_bytes.argtypes = []

@@ -190,6 +190,22 @@ int cubert_op_gemm(const void* X, const void* W, const float* bias, void* Y, int
 int cubert_op_gemm_residual(const void* X, const void* W, const float* bias, const float* R, float* Y,
                             int M, int N, int K, int ldx, int elt, int tile, int flags, void* stream);
 
+/* The same linear with the LayerNorm that follows it in the epilogue as well (cuApplyLayerNorm,
+ * cuda_bert/ops/layernorm.cu:136-206, after op_Linear::forward, ops/linear.cu:91-148):
+ *   Y[M,N] (float32, may be R itself) = LayerNorm(X * W^T + bias + R) * gamma + beta   per row,
+ * eps 1e-12 inside the square root, biased variance; xb (optional) receives a bf16 copy of Y, row-major
+ * or (CUBERT_Y_PACKED) in the packed operand layout.  bf16 operands, tile 256 or 384 (0 = automatic,
+ * which needs a problem large enough for one of them), N a multiple of 256 up to 1024, no split K.
+ * The N / 256 workgroups that hold the same rows exchange partial row sums through `workspace`:
+ * cubert_gemm_layernorm_workspace_bytes(M) bytes of device memory, all zero before the first launch
+ * (a launch leaves it ready for the next one), used by one launch at a time.  A workgroup that waits
+ * for its partners longer than a bounded number of polls gives up and sets the first int of the
+ * workspace to 1. */
+size_t cubert_gemm_layernorm_workspace_bytes(int M);
+int cubert_op_gemm_residual_layernorm(const void* X, const void* W, const float* bias, const float* R,
+                                      const float* gamma, const float* beta, float* Y, void* xb, void* workspace,
+                                      int M, int N, int K, int ldx, int tile, int flags, void* stream);
+
 /* Allocation-free split-K GEMM.  No counterpart in the reference: it is for callers that cannot
  * allocate device memory -- code under hipGraph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  Y[M,N] (float32) = X * W^T + bias, K shared by `splits` (1..16) workgroups per tile,
