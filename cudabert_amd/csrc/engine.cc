@@ -1,5 +1,6 @@
 #include "engine.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <iterator>
@@ -519,7 +520,7 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
     const bool ln_ao = fuse_res && opt_.fuse_layernorm && sp_ao == 1 && gemm_ln_supported(N, H, H, elt);
     const bool ln_fo = fuse_res && opt_.fuse_layernorm && sp_fo == 1 && gemm_ln_supported(N, H, I, elt);
     void* ln_ws = ln_ws_ + (size_t)part * ln_ws_bytes_;
-    if (ln_ao || ln_fo) ln_used_ = true;
+    if (ln_ao || ln_fo) ln_used_ = std::max(ln_used_, part + 1);
 
     if (!mark(kPhEmbed)) return false;
     const bool pk = elt == kBF16;           // packed GEMM operands (weights were packed at load)
@@ -617,11 +618,12 @@ bool Model::classify() {
 
 bool Model::sync() {
     CUBERT_HIP_OK(hipStreamSynchronize(stream_));
-    if (ln_used_) {
+    if (ln_used_ > 0) {
         // A workgroup of a GEMM that normalises in its epilogue gives up after a bounded wait for its
         // partners and raises word 0 of its workspace; the results of that pass are then not valid.
-        ln_used_ = false;
-        for (int i = 0; i < kMaxParts; ++i) {
+        const int parts = ln_used_;
+        ln_used_ = 0;
+        for (int i = 0; i < parts; ++i) {
             int flag = 0;
             CUBERT_HIP_OK(hipMemcpy(&flag, ln_ws_ + (size_t)i * ln_ws_bytes_, sizeof(int), hipMemcpyDeviceToHost));
             if (flag != 0) {

@@ -128,7 +128,7 @@ class Model {
     float* seqpad_ = nullptr;    // padded [B, S, H] sequence output of an unpadded pass
     unsigned char* ln_ws_ = nullptr;   // kMaxParts workspaces of the GEMMs that normalise in their epilogue
     size_t ln_ws_bytes_ = 0;           // size of one of them
-    bool ln_used_ = false;             // such a GEMM ran since sync() last looked at the workspaces' error words
+    int ln_used_ = 0;                  // parts whose workspaces such GEMMs used since sync() last looked at their error words
     bool last_compact_ = false;
     int cur_parts_ = 1;          // parts of the pass being enqueued
     int B_ = 0, S_ = 0;

@@ -34,7 +34,7 @@ struct GemmDev {
     const float* ln_beta;
     unsigned char* ln_xb;                 // bf16 copy of the result (may be null)
     int ln_xb_packed;
-    int* ln_cnt;                          // [0] error flag, [kLnCntFirst + band] arrivals, [.. + ln_bands + band] departures
+    int* ln_cnt;                          // [0] error flag, [1] poll limit (0: default), [kLnCntFirst + band] arrivals, [.. + ln_bands + band] departures
     unsigned long long* ln_stats;         // [row][2 * tiles_n] (sum, sum of squares) as two floats in 64 bits
     int ln_bands;
 };
@@ -451,9 +451,11 @@ __device__ __forceinline__ void gemm_epilogue_ln(const GemmDev& p, f32x16_t (&ac
     int* departures = arrivals + p.ln_bands;
     if (threadIdx.x == 0) {
         __hip_atomic_fetch_add(arrivals, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int wish = p.ln_cnt[1];                         // word 1 of the workspace: the host's own poll limit, if positive
+        const int limit = wish > 0 ? wish : kLnSpinLimit;
         int polls = 0;
         while (__hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p.tiles_n) {
-            if (++polls > kLnSpinLimit) {
+            if (++polls > limit) {
                 __hip_atomic_store(p.ln_cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 break;
             }

@@ -200,7 +200,7 @@ int cubert_op_gemm_residual(const void* X, const void* W, const float* bias, con
  * cubert_gemm_layernorm_workspace_bytes(M) bytes of device memory, all zero before the first launch
  * (a launch leaves it ready for the next one), used by one launch at a time.  A workgroup that waits
  * for its partners longer than a bounded number of polls gives up and sets the first int of the
- * workspace to 1. */
+ * workspace to 1 (the second int, if positive, replaces the built-in poll limit). */
 size_t cubert_gemm_layernorm_workspace_bytes(int M);
 int cubert_op_gemm_residual_layernorm(const void* X, const void* W, const float* bias, const float* R,
                                       const float* gamma, const float* beta, float* Y, void* xb, void* workspace,

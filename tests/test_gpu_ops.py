@@ -633,6 +633,20 @@ def test_gemm_with_residual_and_layernorm_in_the_epilogue(pb, M, N, K, tile, pac
             first = got.copy()
         else:
             assert np.array_equal(first, got)           # the same bits every time
+    # The wait for the partner workgroups is bounded.  With band 0's arrival counter held far below zero its
+    # workgroups can never see it complete: they give up after the poll limit the host puts into word 1 of the
+    # workspace, raise word 0, and the kernel ends normally.
+    if N > 256:
+        ws.zero_()
+        ws[1] = 200
+        ws[64] = -1000000
+        torch.cuda.synchronize()
+        pb.check(pb.lib.cubert_op_gemm_residual_layernorm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Rd.data_ptr(), gd.data_ptr(),
+                                                          bed.data_ptr(), buf[1:].data_ptr(), xb.data_ptr(), ws.data_ptr(), M, N, K, K,
+                                                          tile, gflags, stream()))
+        torch.cuda.synchronize()
+        assert int(ws[0].item()) == 1
+        ws.zero_()
     # refused: tiles other than the two hand-scheduled kernels, N not a multiple of 256, float32 operands are not offered
     assert pb.lib.cubert_op_gemm_residual_layernorm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Rd.data_ptr(), gd.data_ptr(),
                                                     bed.data_ptr(), buf[1:].data_ptr(), xb.data_ptr(), ws.data_ptr(), M, N, K, K,
