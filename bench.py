@@ -441,7 +441,7 @@ def main():
         emb_bytes = N * (12 + H * 4 + H * 4) + (S + 2) * H * 4 + 2 * H * 4
         # bf16 mode, large batches: the LayerNorm runs in the epilogue of the GEMM before it
         ln_in_gemm = (e == 2 and os.environ.get("CUBERT_FUSE_LAYERNORM", "1") != "0" and
-                      os.environ.get("CUBERT_FUSE_RESIDUAL", "1") != "0" and H % 256 == 0 and N >= 4096)
+                      os.environ.get("CUBERT_FUSE_RESIDUAL", "1") != "0" and H % 256 == 0 and N >= 6144)
         # fused attention reads q, k, v^T and the mask rows and writes the context: its HBM bytes
         att_bytes = ((3.0 * N * H + 1.0 * N * H) * e + B * A * 64 * (Sp - S) * e + 4.0 * B * Sp) * L
         phases = {}

@@ -39,6 +39,7 @@ namespace cubert {
 bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
 bool launch_gemm_bf16_t256x128(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
 int gemm_pick_tile(int M, int N, int K, int elt);
+int gemm_ln_pick_tile(int M, int N, int K, int elt);
 
 namespace {
 
@@ -290,11 +291,18 @@ namespace {
 bool ln_shape_ok(int N, int K, int elt) { return elt == kBF16 && N > 0 && N % 256 == 0 && N <= 1024 && K % 32 == 0 && K >= 64; }
 }  // namespace
 
-bool gemm_ln_supported(int M, int N, int K, int elt) {
-    if (M <= 0 || !ln_shape_ok(N, K, elt)) return false;
-    const int bt = gemm_pick_tile(M, N, K, elt);
-    return bt == kTile256x128 || (bt == 256 && K % 128 == 0);
+// Tile of a GEMM with the LayerNorm in its epilogue, 0 if the separate kernels are the better choice.
+// Measured on MI355X (N = 768 and 1024, K = N and 4 N): from about 6000 rows on the fused kernel beats
+// GEMM + LayerNorm launch.  Inside a forward pass (two half-batches on two streams) the 256 x 256 tile wins
+// once its tiles cover half of the CUs (152 and 200 tiles: +7 % on the pass over the 256 x 128 tile), below
+// that the 256 x 128 tile, two workgroups per CU and half as coarse (96 tiles: +3 %).
+int gemm_ln_pick_tile(int M, int N, int K, int elt) {
+    if (M < 6144 || !ln_shape_ok(N, K, elt)) return 0;
+    const long tiles256 = (long)((M + 255) / 256) * (N / 256);
+    return (K % 128 == 0 && tiles256 >= 128) ? 256 : kTile256x128;
 }
+
+bool gemm_ln_supported(int M, int N, int K, int elt) { return gemm_ln_pick_tile(M, N, K, elt) != 0; }
 
 int gemm_pick_tile(int M, int N, int K, int elt) {
     auto tiles = [&](int bt) { return (long)((M + bt - 1) / bt) * ((N + bt - 1) / bt); };
@@ -416,9 +424,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         }
     }
     int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
-    // With the LayerNorm in the epilogue the 256 x 256 tile measured faster than 256 x 128 wherever both apply
-    // (one exchange per 256 rows instead of two, and the long epilogue does not share the CU's LDS pipe).
-    if (epi == kEpiBiasResLN && !p.tile && p.K % 128 == 0) bt = 256;
+    if (epi == kEpiBiasResLN && !p.tile) bt = gemm_ln_pick_tile(p.M, p.N, p.K, p.elt);
     if (d.splits > 1 && bt == 256 && !p.tile) bt = 128;      // the hand-scheduled kernel does not split
     if (epi == kEpiBiasResLN && p.compiler_scheduled) { set_error("gemm: the LayerNorm epilogue has no compiler-scheduled kernel"); return false; }
     if (bt == kTile256x128) {
