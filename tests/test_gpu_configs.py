@@ -179,6 +179,33 @@ def test_cfg3_large_latency_regime_graph_and_split_k(pb, large_ckpt, monkeypatch
         pb.unload_model(m_nosplit)
 
 
+def test_layernorm_in_gemm_epilogue_inside_a_captured_graph(pb, base_ckpt):
+    """A batch just below the hipGraph limit (32 x 200 = 6400 tokens) is large enough for the GEMMs that
+    normalise in their epilogue: their workgroups count themselves in and out on words of a workspace that
+    every launch has to leave at zero, replays of the captured graph included.  Eager, capture, replays: the
+    same bits each time, the first sequences within tolerance of the oracle."""
+    D = W.BASE
+    B, S = 32, 200
+    lens = np.random.default_rng(3).integers(60, S + 1, size=B)
+    lens[0] = S
+    ids, seg, mask = synth.make_inputs(B, S, list(lens), seed=77)
+    m = load(pb, D, base_ckpt.bf16x, BF16, B, S, graph=8192)
+    try:
+        first = None
+        for call in range(5):
+            pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+            if first is None:
+                first = (pooled, seq)
+            else:
+                assert np.array_equal(pooled, first[0]) and np.array_equal(seq, first[1]), call
+        assert pb.lib.cubert_graphs_cached(m) == 1
+    finally:
+        pb.unload_model(m)
+    n = 2
+    seq_ref, pooled_ref = O.forward_torch(base_ckpt.npy_bf16x, D.heads, ids[:n], seg[:n], mask[:n])
+    assert err(first[1][:n], seq_ref) < TOL[BF16] and err(first[0][:n], pooled_ref) < TOL[BF16]
+
+
 # ------------------------------------------------------------------ configuration 4 ----
 
 def test_cfg4_large_b64_s512_skewed(pb, large_ckpt):
