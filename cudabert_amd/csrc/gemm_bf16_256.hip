@@ -152,6 +152,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
     const int xb = lds_base + (wm * 64 + l32) * 64 + ((g ^ sw) << 4);       // + 0x4000 is in the read offsets
     const int m0b = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
     const int ht = p.K / 32;
+    const int wkmax = (ht - 1) * wkstep, xkmax = (ht - 1) * xkstep;      // K offset of the last tile
 
     f32x16_t acc[4][2];       // zeroed inside the asm block
 
@@ -159,7 +160,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_t256x128_kernel(const GemmDe
 #include "gemm_bf16_256x128_loop.inc"
         : CUBERT_ACC_OPERANDS_H
         : [wb] "v"(wb), [xb] "v"(xb), [wv0] "v"(w_v0), [xv0] "v"(x_v0), [wres] "s"(wres), [xres] "s"(xres),
-          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep)
+          [w64] "s"(w64), [x64] "s"(x64), [ht] "s"(ht), [m0b] "s"(m0b), [wkstep] "s"(wkstep), [xkstep] "s"(xkstep),
+          [wkmax] "s"(wkmax), [xkmax] "s"(xkmax)
         : "memory", "scc", "m0", "s92", "s93", "s94", "s96", "s97", "s98", "v64", "v65", "v66", "v67", "v68", "v69",
           CUBERT_V10(7), CUBERT_V10(8), CUBERT_V10(9), CUBERT_V10(10), CUBERT_V10(11), "v120", "v121", "v122",
           "v123", "v124", "v125");

@@ -238,7 +238,7 @@ def main():
 # k-phase 1, read a half-step ago; 8 MFMAs on A with the 6 reads of this tile's k-phase 1
 # (into B) behind them; the 6 global->LDS loads of tile h+2 spread behind the MFMAs;
 # vmcnt(6) (everything but the loads just issued, i.e. tile h+1, has landed); barrier.  Loads
-# issued for tiles past the end of K fetch valid memory or zeros and are never used; the
+# issued for tiles past the end of K fetch the last tile again and are never used; the
 # block ends with vmcnt(0) and a barrier so that nothing lands in the LDS afterwards.
 H_WA, H_XA, H_WB, H_XB = 64, 80, 88, 104
 H_BASE, H_CUR = 112, 122
@@ -285,6 +285,14 @@ def main_half():
         e.emit("s_cselect_b32 s%d, 0, s%d" % (reg, reg))
 
     e.emit("; ======== prologue: tiles 0, 1 -> stages 0, 1 ========")
+    def advance_k_clamped():
+        # The loads run two tiles ahead of the multiply, so the last two half-steps ask for tiles
+        # past the end of K: they fetch the last tile again (the range check of a buffer
+        # descriptor does not cover the scalar offset, so the offset itself has to stay inside).
+        advance_k(e)
+        e.emit("s_min_u32 s96, s96, %[wkmax]")
+        e.emit("s_min_u32 s98, s98, %[xkmax]")
+
     for t in range(2):
         for k in range(6):
             m0, ld = dma(k)
@@ -292,7 +300,7 @@ def main_half():
             e.emit("s_nop 0")
             e.emit(ld)
         rotate(93)
-        advance_k(e)
+        advance_k_clamped()
     e.emit("s_waitcnt vmcnt(6)")           # tile 0 has landed
     e.emit("s_barrier")
 
@@ -330,7 +338,7 @@ def main_half():
     def end_of_half_step():
         rotate(92)
         rotate(93)
-        advance_k(e)
+        advance_k_clamped()
         # vmcnt(6): everything but the loads just issued, i.e. the next tile, has landed.
         # lgkmcnt(0): my reads of this tile are done before anybody may overwrite its stage.
         e.emit("s_waitcnt vmcnt(6) lgkmcnt(0)")
