@@ -85,8 +85,9 @@ def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[precision], 4),
                 "avg_launch_ms": round(k_ms, 4), "flop_per_launch": flops_per_launch,
                 "traffic": measured_traffic(precision, N, I, H)[0],
-                "traffic_source": "profiles/ffn_in_gemm_cfg2_bf16_pmc.txt (rocprofv3 --pmc, commit %s)" %
-                                  measured_traffic(precision, N, I, H)[1]}
+                "traffic_source": ("profiles/ffn_in_gemm_cfg2_bf16_pmc.txt (rocprofv3 --pmc, commit %s)" %
+                                   measured_traffic(precision, N, I, H)[1])
+                                  if measured_traffic(precision, N, I, H)[0] is not None else None}
     del X, Wt, Y
     return roofline
 

@@ -27,6 +27,8 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 
 template <int ELT>
 __global__ __launch_bounds__(256) void attention_kernel(
@@ -193,6 +195,15 @@ __global__ __launch_bounds__(256) void attention_kernel(
 // visible key in the row their probabilities are exactly zero in float32
 // (exp2 of less than -14000), so the result is bit-identical to walking them.
 // If no key at all is visible nothing is skipped.
+//
+// VROW: V arrives as [S, 64] rows like K (the QKV GEMM then stores it in whole row segments instead
+// of two bytes at a time).  It sits in the LDS as rows of 128 bytes whose four 32-byte blocks are
+// permuted by (row >> 1) & 3, and the transposition the second MFMA needs happens in the read:
+// ds_read_b64_tr_b16 hands lane i of a group of 16 the i-th 16-bit element of each of the four
+// 32-byte pieces that lanes 4r .. 4r+3 (r = 0..3) point at, so with piece r = 16 features of key
+// kb + r a lane receives its feature for four consecutive keys.  The block permutation puts the
+// four pieces of a group into four different bank ranges.
+template <bool VROW>
 __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
     const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
@@ -201,7 +212,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* sK = smem;
     unsigned char* sV = smem + (size_t)Sp * 128;
-    float* sM = reinterpret_cast<float*>(sV + 64 * (size_t)vstride);
+    float* sM = reinterpret_cast<float*>(sV + (VROW ? (size_t)Sp * 128 : 64 * (size_t)vstride));
     int* sLive = reinterpret_cast<int*>(sM + Sp);
 
     const int tid = threadIdx.x, nthr = blockDim.x;
@@ -212,7 +223,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const size_t bh = (size_t)b * heads + h;
     const unsigned char* qb = q + bh * S * 128;
     const unsigned char* kb = k + bh * S * 128;
-    const unsigned char* vb = vt + bh * 64 * (size_t)Sp * 2;
+    const unsigned char* vb = vt + (VROW ? bh * S * 128 : bh * 64 * (size_t)Sp * 2);
 
     // ---- stage K (rows S..Sp-1 zero), V^T and the mask row ----
     // The workgroup has 2 Sp threads, K is 8 Sp and V^T 8 Sp 16-byte chunks: four of each per
@@ -230,9 +241,16 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int c = tid + i * nthr;
-        vrow_i[i] = c / vchunks;
-        vch_i[i] = c - vrow_i[i] * vchunks;
-        vd[i] = *reinterpret_cast<const uint4*>(vb + ((size_t)vrow_i[i] * Sp + vch_i[i] * 8) * 2);
+        if constexpr (VROW) {
+            vrow_i[i] = c >> 3;
+            vch_i[i] = c & 7;
+            vd[i] = make_uint4(0u, 0u, 0u, 0u);
+            if (vrow_i[i] < S) vd[i] = *reinterpret_cast<const uint4*>(vb + (size_t)c * 16);
+        } else {
+            vrow_i[i] = c / vchunks;
+            vch_i[i] = c - vrow_i[i] * vchunks;
+            vd[i] = *reinterpret_cast<const uint4*>(vb + ((size_t)vrow_i[i] * Sp + vch_i[i] * 8) * 2);
+        }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -242,9 +260,14 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        uint2* dst = reinterpret_cast<uint2*>(sV + (size_t)vrow_i[i] * vstride + vch_i[i] * 16);     // rows are 8-byte aligned
-        dst[0] = make_uint2(vd[i].x, vd[i].y);
-        dst[1] = make_uint2(vd[i].z, vd[i].w);
+        if constexpr (VROW) {
+            const int row = vrow_i[i], ch = vch_i[i];
+            *reinterpret_cast<uint4*>(sV + row * 128 + ((((ch >> 1) ^ ((row >> 1) & 3)) << 5) | ((ch & 1) << 4))) = vd[i];
+        } else {
+            uint2* dst = reinterpret_cast<uint2*>(sV + (size_t)vrow_i[i] * vstride + vch_i[i] * 16);     // rows are 8-byte aligned
+            dst[0] = make_uint2(vd[i].x, vd[i].y);
+            dst[1] = make_uint2(vd[i].z, vd[i].w);
+        }
     }
     {
         // wave w looks at mask block w
@@ -286,6 +309,16 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
         for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
     float run_max = -INFINITY, run_sum = 0.0f;
     const int ksw = l32 & 7;
+    // VROW: where my 8-byte piece of a transposing read lies for key block 0, f = 0, per feature block db.
+    // Row 4 g + (i >> 2), i = l32 & 15; logical 32-byte block 2 db + (l32 >> 4), permuted by (row >> 1) & 3,
+    // which the multiples of 8 that k0, f and the second read add to the row do not change.
+    const unsigned char* vpiece[2];
+    {
+        const int i16 = l32 & 15, prow = 4 * g + (i16 >> 2), psw = (prow >> 1) & 3;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+            vpiece[db] = sV + prow * 128 + (((2 * db + (l32 >> 4)) ^ psw) << 5) + (i16 & 3) * 8;
+    }
 
     for (int kblk = 0; kblk < nblk; ++kblk) {
         if (!((live >> kblk) & 1u)) continue;
@@ -364,11 +397,22 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
             for (int e = 0; e < 8; ++e) pf[e] = (__bf16)sc[8 * f + e];
 #pragma unroll
             for (int db = 0; db < 2; ++db) {
-                const unsigned char* vrow = sV + (size_t)(32 * db + l32) * vstride + (k0 + 16 * f + 4 * g) * 2;
-                const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-                const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
-                const uint4 vf = {lo.x, lo.y, hi.x, hi.y};
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf), pf, o[db], 0, 0, 0);
+                if constexpr (VROW) {
+                    // my piece: 4 features of key k0 + 16 f + 4 g + (i >> 2) (and of the key 8 further), i = l32 & 15
+                    const unsigned char* piece = vpiece[db] + (k0 + 16 * f) * 128;
+                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        reinterpret_cast<__attribute__((address_space(3))) s16x4_t*>((__attribute__((address_space(3))) unsigned char*)piece));
+                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        reinterpret_cast<__attribute__((address_space(3))) s16x4_t*>((__attribute__((address_space(3))) unsigned char*)(piece + 8 * 128)));
+                    const s16x8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf), pf, o[db], 0, 0, 0);
+                } else {
+                    const unsigned char* vrow = sV + (size_t)(32 * db + l32) * vstride + (k0 + 16 * f + 4 * g) * 2;
+                    const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                    const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                    const uint4 vf = {lo.x, lo.y, hi.x, hi.y};
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf), pf, o[db], 0, 0, 0);
+                }
             }
         }
     }
@@ -397,7 +441,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
                       bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream,
-                      const int* cu) {
+                      const int* cu, bool v_rowmajor) {
     if (ctx_packed && elt != kBF16) { set_error("attention: only a bf16 context can be packed"); return false; }
     const int cp = ctx_packed ? 1 : 0;
     if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
@@ -420,7 +464,7 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
     unsigned char* cc = static_cast<unsigned char*>(ctx);
     if (elt == kBF16 && S <= 512) {
         const int vstride = round_up(Sp * 2, 256) + 8;
-        const size_t lds = (size_t)Sp * 128 + 64 * (size_t)vstride + (size_t)Sp * 4 + 64;
+        const size_t lds = (size_t)Sp * 128 + (v_rowmajor ? (size_t)Sp * 128 : 64 * (size_t)vstride) + (size_t)Sp * 4 + 64;
         // More than 64 KiB of dynamic LDS has to be allowed once per device.
         // (Several host threads, one model each, may get here together: the flag is atomic and
         // setting the attribute twice is harmless.)
@@ -428,15 +472,22 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
         int dev = 0;
         CUBERT_HIP_OK(hipGetDevice(&dev));
         if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
-            CUBERT_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_lds_kernel),
+            CUBERT_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_lds_kernel<false>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            CUBERT_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_lds_kernel<true>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
         }
-        hipLaunchKernelGGL(attention_lds_kernel, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd, cc,
-                           heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);
+        if (v_rowmajor)
+            hipLaunchKernelGGL(attention_lds_kernel<true>, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd,
+                               cc, heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);
+        else
+            hipLaunchKernelGGL(attention_lds_kernel<false>, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd,
+                               cc, heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);
         CUBERT_HIP_OK(hipGetLastError());
         return true;
     }
+    if (v_rowmajor) { set_error("attention: a row-major V needs bf16 operands and S <= 512"); return false; }
     dim3 grid((S + 127) / 128, heads, B), block(256);
     if (elt == kBF16)
         hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu);

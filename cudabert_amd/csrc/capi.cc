@@ -59,6 +59,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.split_k = env_int("CUBERT_SPLIT_K", 1) != 0;
     opt.fuse_residual = env_int("CUBERT_FUSE_RESIDUAL", 1) != 0;
     opt.fuse_layernorm = env_int("CUBERT_FUSE_LAYERNORM", 1) != 0;
+    opt.v_rowmajor = env_int("CUBERT_V_ROWMAJOR", 1) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;
@@ -319,7 +320,7 @@ int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q,
     cubert::GemmParams p;
     p.X = X; p.W = W; p.bias = bias; p.M = B * S; p.N = 3 * heads * 64; p.K = heads * 64; p.ldx = heads * 64;
     p.elt = elt; p.epilogue = cubert::kEpiQKV; p.q = q; p.k = k; p.vt = vt; p.S = S; p.Sp = cubert::round_up(S, 32);
-    p.heads = heads; p.tile = tile;
+    p.heads = heads; p.tile = tile; p.v_rowmajor = (flags & CUBERT_V_ROWMAJOR) != 0;
     apply_gemm_flags(&p, flags);
     return cubert::launch_gemm(p, static_cast<hipStream_t>(stream)) ? 0 : 1;
 }
@@ -332,7 +333,7 @@ int cubert_op_attention(const void* q, const void* k, const void* vt, const floa
     cubert::set_error("");
     return cubert::launch_attention(q, k, vt, maskadd, ctx, (flags & CUBERT_Y_PACKED) != 0, B, heads, S,
                                     cubert::round_up(S > 0 ? S : 1, 32), scale, elt,
-                                    static_cast<hipStream_t>(stream)) ? 0 : 1;
+                                    static_cast<hipStream_t>(stream), nullptr, (flags & CUBERT_V_ROWMAJOR) != 0) ? 0 : 1;
 }
 
 int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta, void* xb,

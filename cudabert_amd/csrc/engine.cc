@@ -531,14 +531,17 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
         const LayerDev& L = layers_[i];
         GemmParams g;
         g.elt = elt;
-        // QKV projection, scattered per head (V transposed)
+        // QKV projection, scattered per head (V transposed, unless the attention kernel that follows
+        // transposes on its own LDS reads)
+        const bool vrow = opt_.v_rowmajor && elt == kBF16 && S <= 512;
         g.X = xin; g.ldx = H; g.W = L.w_qkv; g.bias = L.b_qkv; g.M = N; g.N = 3 * H; g.K = H;
         g.epilogue = kEpiQKV; g.q = q; g.k = k; g.vt = vt; g.S = S; g.Sp = Sp; g.heads = D.heads;
+        g.v_rowmajor = vrow;
         g.rowmap = cp ? cp->rowmap : nullptr;
         g.x_packed = g.w_packed = pk;
         if (!mark(kPhQKV) || !launch_gemm(g, st)) return false;
         if (!mark(kPhAttention)) return false;
-        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st, cu)) return false;
+        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;

@@ -28,6 +28,7 @@ struct ModelOptions {
     int split_min_tokens = 8192;   // batches of at least this many tokens run as two halves on two streams (0: never)
     bool fuse_residual = true;     // residual add in the epilogue of the GEMM before each LayerNorm
     bool fuse_layernorm = true;    // ... and the LayerNorm itself, where the GEMM kernel supports it (bf16, large batches)
+    bool v_rowmajor = true;        // bf16, S <= 512: V is stored [B, heads, S, 64] like K; attention transposes on its LDS reads
     bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
     int varlen = -1;               // host-input calls with prefix masks compute only the valid tokens: 1 always,
                                    // 0 never, -1 when the caller asks for no sequence output (see forward_host)

@@ -404,6 +404,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         d.q = static_cast<unsigned char*>(p.q);
         d.k = static_cast<unsigned char*>(p.k);
         d.vt = static_cast<unsigned char*>(p.vt);
+        d.v_rowmajor = p.v_rowmajor ? 1 : 0;
         d.S = p.S; d.Sp = p.Sp; d.heads = p.heads; d.hidden = p.heads * 64;
         d.rowmap = p.rowmap;
         d.y_packed = 0;

@@ -27,6 +27,7 @@ struct GemmDev {
     int x_packed, w_packed, y_packed;     // operand / result in the packed layout (common.h)
     int xn_parts;                         // how the XCDs divide the tile grid (tile_of_block)
     const int* rowmap;                    // QKV epilogue: row m -> token b * S + s (nullptr: m itself)
+    int v_rowmajor;                       // QKV epilogue: V is stored like q / k instead of transposed
     const float* R;                       // kEpiBiasRes: [M, N] float32 row-major, added to the result
     int splits;                           // split K: blockIdx.y owns a K range, results go to Y + y * M * N (f32)
     // kEpiBiasResLN: LayerNorm in the epilogue (gemm_epilogue_ln)
@@ -267,7 +268,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
                     v[e] = t;
                 }
                 if constexpr (EPI == kEpiQKV || EPI == kEpiQKVMap) {
-                    if (n >= 2 * p.hidden) {
+                    if (n >= 2 * p.hidden && !p.v_rowmajor) {
                         if (m < p.M && n < p.N) {
                             const int hn = n - 2 * p.hidden;
                             const size_t bh = (size_t)bidx * p.heads + (hn >> 6);
@@ -309,12 +310,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             if constexpr (EPI == kEpiQKVMap) tok = __shfl(tokj[j], row);      // before any lane leaves
             if (mm >= p.M || n >= p.N) continue;
             if constexpr (EPI == kEpiQKV || EPI == kEpiQKVMap) {
-                if (n >= 2 * p.hidden) continue;
+                if (n >= 2 * p.hidden && !p.v_rowmajor) continue;           // left transposed, straight from the accumulators
                 const int b2 = tok / p.S, s2 = tok - b2 * p.S;
-                const int which = n >= p.hidden ? 1 : 0;
+                const int which = n >= 2 * p.hidden ? 2 : n >= p.hidden ? 1 : 0;
                 const int hn = n - which * p.hidden;
                 const size_t bh = (size_t)b2 * p.heads + (hn >> 6);
-                *reinterpret_cast<u32x4_t*>((which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES) = d;
+                *reinterpret_cast<u32x4_t*>((which == 2 ? p.vt : which ? p.k : p.q) + ((bh * p.S + s2) * 64 + (hn & 63)) * OES) = d;
             } else if (p.y_packed) {
                 // packed bf16 result: the next GEMM's activation operand
                 *reinterpret_cast<u32x4_t*>(p.Y + packed_offset(mm, n * 2, p.N * 2 / 64)) = d;

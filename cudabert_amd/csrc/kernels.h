@@ -54,6 +54,7 @@ struct GemmParams {
     void* q = nullptr;
     void* k = nullptr;
     void* vt = nullptr;
+    bool v_rowmajor = false;  // kEpiQKV: V leaves like q and k, [B, heads, S, 64], instead of transposed (bf16 attention with S <= 512 transposes on its LDS reads)
     int S = 0, Sp = 0, heads = 0;
     const int* rowmap = nullptr;   // kEpiQKV on compact rows: row m is token rowmap[m] = b * S + s
     // kEpiBias with a float32 row-major Y: [M, N] float32 added to the result (the residual branch of
@@ -99,7 +100,8 @@ bool gemm_ln_supported(int M, int N, int K, int elt);
 // ctx_packed (bf16 only): write ctx in the packed GEMM-operand layout (common.h).
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd,
                       void* ctx, bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt,
-                      hipStream_t stream, const int* cu = nullptr);
+                      hipStream_t stream, const int* cu = nullptr, bool v_rowmajor = false);
+// v_rowmajor (bf16, S <= 512 only): `vt` holds V as [B, heads, S, 64] like k.
 
 // ----------------------------------------------------------- LayerNorm -----
 // x <- LayerNorm(x + y) * gamma + beta   over rows of length H, in place on the

@@ -169,6 +169,8 @@ long cubert_capacity_tokens(void* model);
 #define CUBERT_Y_PACKED 4           /* write Y packed (bf16 output only) */
 #define CUBERT_COMPILER_SCHEDULED 8 /* 256 tile: general kernel instead of the hand-scheduled one */
 #define CUBERT_LN_NO_RESIDUAL 16    /* cubert_op_add_layernorm: y already contains the residual stream */
+#define CUBERT_V_ROWMAJOR 32        /* cubert_op_gemm_qkv / cubert_op_attention (bf16, S <= 512): the `vt` argument holds V as
+                                       [B, heads, S, 64] like k instead of transposed */
 /* Split K (cubert_op_gemm, epilogue 0, float32 Y): n workgroups share a tile, each reduces 1/n of K
  * and writes its partial sum to Y + i * M * N (the bias is in partial 0); Y holds n * M * N floats and
  * the consumer adds the parts (cubert_op_add_layernorm takes the count in the same flag bits). */
@@ -223,7 +225,7 @@ size_t cubert_noalloc_scratch_bytes(void);
 
 /* Fused QKV projection (op_BatchedLinear::forward, cuda_bert/ops/linear.cu:241-319):
  * X[B*S, hidden] * Wqkv[3*hidden, hidden]^T + bias -> q,k [B,heads,S,64],
- * vt [B,heads,64,Sp] with Sp = S rounded up to 32. */
+ * vt [B,heads,64,Sp] with Sp = S rounded up to 32 (CUBERT_V_ROWMAJOR: V as [B,heads,S,64] in the same buffer). */
 int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q, void* k, void* vt,
                        int B, int S, int heads, int elt, int tile, int flags, void* stream);
 
@@ -231,7 +233,7 @@ int cubert_op_gemm_qkv(const void* X, const void* W, const float* bias, void* q,
  * cuda_bert/ops/batch_matmul.cu:48-141, ops/softmax.cu:86-143). */
 int cubert_op_attention(const void* q, const void* k, const void* vt, const float* maskadd,
                         void* ctx, int B, int heads, int S, float scale, int elt, int flags,
-                        void* stream); /* flags: CUBERT_Y_PACKED writes ctx packed (bf16) */
+                        void* stream); /* flags: CUBERT_Y_PACKED writes ctx packed (bf16); CUBERT_V_ROWMAJOR */
 
 /* x <- LayerNorm(x + y); optional bf16 copy xb (op_LayerNorm::forward,
  * cuda_bert/ops/layernorm.cu:136-206). */

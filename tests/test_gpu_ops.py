@@ -9,6 +9,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 F32, BF16 = 0, 1
+V_ROWMAJOR = 32          # CUBERT_V_ROWMAJOR
 
 
 @pytest.fixture(scope="module")
@@ -139,8 +140,9 @@ def test_gemm_rejects_bad_shapes(pb):
 @pytest.mark.parametrize("elt", [F32, BF16])
 @pytest.mark.parametrize("B,S,heads,tile", [(3, 33, 2, 64), (2, 200, 4, 128), (5, 128, 12, 256), (2, 200, 4, 384),
                                             (5, 128, 12, 384)])
-def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile):
-    print("qkv", elt, B, S, heads, tile, flush=True)
+@pytest.mark.parametrize("v_rowmajor", [0, 1])
+def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile, v_rowmajor):
+    print("qkv", elt, B, S, heads, tile, v_rowmajor, flush=True)
     if tile == 384 and elt == F32:
         pytest.skip("the 256 x 128 kernel is bf16 only")
     rng = np.random.default_rng(B + S)
@@ -161,11 +163,18 @@ def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile):
     k = torch.zeros_like(q)
     vt = torch.zeros((B, heads, 64, Sp), dtype=tdt, device="cuda")
     pb.check(pb.lib.cubert_op_gemm_qkv(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), q.data_ptr(), k.data_ptr(),
-                                       vt.data_ptr(), B, S, heads, elt, tile, 0, stream()))
+                                       vt.data_ptr(), B, S, heads, elt, tile, V_ROWMAJOR if v_rowmajor else 0, stream()))
     torch.cuda.synchronize()
     tol = 2e-4 if elt == F32 else 3e-2
     assert np.abs(q.float().cpu().numpy() - q_ref).max() < tol
     assert np.abs(k.float().cpu().numpy() - k_ref).max() < tol
+    if v_rowmajor:
+        # V like q and k, [B, heads, S, 64], at the start of the same buffer; the rest stays untouched
+        flat = vt.float().cpu().numpy().reshape(-1)
+        n = B * heads * S * 64
+        assert np.abs(flat[:n].reshape(B, heads, S, 64) - vt_ref.transpose(0, 1, 3, 2)).max() < tol
+        assert (flat[n:] == 0).all()
+        return
     vt_h = vt.float().cpu().numpy()
     assert np.abs(vt_h[..., :S] - vt_ref).max() < tol
     assert (vt_h[..., S:] == 0).all()                    # padding columns untouched
@@ -210,6 +219,17 @@ def test_attention(pb, elt, B, S, heads):
     torch.cuda.synchronize()
     got = ctx.float().cpu().numpy()
     assert np.isfinite(got).all()
+    if elt == BF16:
+        # V handed over as [B, heads, S, 64]: the kernel transposes on its LDS reads; same bits
+        vr = dev(v, tdt)
+        ctx2 = torch.full((B * S, heads * 64), float("nan"), dtype=tdt, device="cuda")
+        pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vr.data_ptr(), md.data_ptr(), ctx2.data_ptr(),
+                                            B, heads, S, scale, elt, V_ROWMAJOR, stream()))
+        torch.cuda.synchronize()
+        assert torch.equal(ctx.view(torch.int16), ctx2.view(torch.int16))
+    else:
+        assert pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), ctx.data_ptr(),
+                                          B, heads, S, scale, elt, V_ROWMAJOR, stream()) != 0      # bf16 only
     tol = 2e-5 * 10 if elt == F32 else 2e-2
     err = np.abs(got - ref).reshape(B, S, -1).max(axis=(1, 2))
     for b in range(B):
@@ -497,6 +517,12 @@ def test_attention_random_shapes(pb):
         got = ctx.float().cpu().numpy()
         assert np.isfinite(got).all(), case
         assert np.abs(got - ref).max() < 2e-2, (case, np.abs(got - ref).max())
+        vr = dev(v, torch.bfloat16)
+        ctx2 = torch.full((B * S, heads * 64), float("nan"), dtype=torch.bfloat16, device="cuda")
+        pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vr.data_ptr(), md.data_ptr(), ctx2.data_ptr(),
+                                            B, heads, S, 0.125, BF16, V_ROWMAJOR, stream()))
+        torch.cuda.synchronize()
+        assert torch.equal(ctx.view(torch.int16), ctx2.view(torch.int16)), case
 
 
 LN_NO_RESIDUAL = 16
