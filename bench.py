@@ -352,14 +352,16 @@ def main():
         Sp = (S + 31) // 32 * 32
         q = torch.randn((B, A, S, 64), device="cuda").to(tdt)
         k = torch.randn((B, A, S, 64), device="cuda").to(tdt)
-        vt = torch.randn((B, A, 64, Sp), device="cuda").to(tdt)
+        vrow = prec == pybert.BF16 and S <= 512       # as in the model: V head-major like k, transposed by the kernel's LDS reads
+        vt = torch.randn((B, A, S, 64) if vrow else (B, A, 64, Sp), device="cuda").to(tdt)
         madd = np.full((B, Sp), -np.inf, np.float32)
         madd[:, :S] = (1.0 - mask.astype(np.float32)) * -10000.0
         madd = torch.from_numpy(madd).cuda()
         ctx = torch.empty((rows, H), dtype=tdt, device="cuda")
         for _ in range(20):
             pybert.check(lib.cubert_op_attention(q.data_ptr(), k.data_ptr(), vt.data_ptr(), madd.data_ptr(), ctx.data_ptr(),
-                                                 B, A, S, 0.125, prec, 4 if prec == pybert.BF16 else 0, st.cuda_stream))
+                                                 B, A, S, 0.125, prec, (4 if prec == pybert.BF16 else 0) | (32 if vrow else 0),
+                                                 st.cuda_stream))
         a = torch.empty(64 << 20, dtype=torch.float32, device="cuda")     # 256 MiB read + 256 MiB written
         c = torch.empty_like(a)
         for _ in range(3):
@@ -443,8 +445,10 @@ def main():
         # bf16 mode, large batches: the LayerNorm runs in the epilogue of the GEMM before it
         ln_in_gemm = (e == 2 and os.environ.get("CUBERT_FUSE_LAYERNORM", "1") != "0" and
                       os.environ.get("CUBERT_FUSE_RESIDUAL", "1") != "0" and H % 256 == 0 and N >= 6144)
-        # fused attention reads q, k, v^T and the mask rows and writes the context: its HBM bytes
-        att_bytes = ((3.0 * N * H + 1.0 * N * H) * e + B * A * 64 * (Sp - S) * e + 4.0 * B * Sp) * L
+        # fused attention reads q, k, v and the mask rows and writes the context: its HBM bytes (a transposed V,
+        # fp32 mode or S > 512, is padded to Sp key columns)
+        v_pad = 0 if (e == 2 and S <= 512 and os.environ.get("CUBERT_V_ROWMAJOR", "1") != "0") else B * A * 64 * (Sp - S) * e
+        att_bytes = ((3.0 * N * H + 1.0 * N * H) * e + v_pad + 4.0 * B * Sp) * L
         phases = {}
         for i, name in enumerate(pybert.PHASES):
             ms = float(acc[i])
