@@ -88,6 +88,26 @@ def roofline_leg(torch, pybert, lib, prec, precision, N, I, H):
                 "traffic_source": ("profiles/ffn_in_gemm_cfg2_bf16_pmc.txt (rocprofv3 --pmc, commit %s)" %
                                    measured_traffic(precision, N, I, H)[1])
                                   if measured_traffic(precision, N, I, H)[0] is not None else None}
+    # Yardstick, not part of the product: the vendor library's plain GEMM (torch.matmul: no bias, no
+    # GELU, row-major operands) on the same shape and the same kind of data, timed the same way.
+    try:
+        Xr = torch.randn((N, H), device="cuda").to(tdt)
+        Wr = (torch.randn((H, I), device="cuda") * 0.02).to(tdt)
+        for _ in range(20):
+            torch.matmul(Xr, Wr)
+        e0.record(st)
+        for _ in range(launches):
+            torch.matmul(Xr, Wr)
+        e1.record(st)
+        e1.synchronize()
+        v_ms = e0.elapsed_time(e1) / launches
+        roofline["vendor_library_same_shape"] = {
+            "what": "torch.matmul %dx%dx%d %s, no epilogue, %d launches back to back" % (N, I, H, precision, launches),
+            "avg_launch_ms": round(v_ms, 4), "achieved": round(flops_per_launch / v_ms / 1e9, 1),
+            "frac": round(flops_per_launch / v_ms / 1e9 / PEAK_TFLOPS[precision], 4)}
+        del Xr, Wr
+    except RuntimeError as err:            # a yardstick only: its failure must not take the record down
+        roofline["vendor_library_same_shape"] = {"error": str(err)[:200]}
     del X, Wt, Y
     return roofline
 
@@ -522,6 +542,7 @@ def main():
                          "measured": "HIP events around each of the %d FFN-in launches of a forward pass, 3 passes" % L,
                          "standalone_back_to_back": {"launches": 50, "avg_launch_ms": standalone["avg_launch_ms"],
                                                      "achieved": standalone["achieved"], "frac": standalone["frac"]}})
+    # (vendor_library_same_shape compares with standalone_back_to_back: both are 50 launches on their own)
     ops = standalone_ops(torch, pybert, mask, B, S, H, A)
     # With the LayerNorm inside two of the GEMMs their phase times are not GEMM-only any more; the same
     # profile of a model that launches the LayerNorm kernel keeps the pure GEMM figures comparable.
