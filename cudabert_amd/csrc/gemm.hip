@@ -185,15 +185,31 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
         CUBERT_ISSUE_TILE(NEXT, (kt) + NS - 1);                                                             \
         int wb = woff0, xb = xoff0;                                                                         \
         asm volatile("" : "+v"(wb), "+v"(xb));                                                              \
-        u32x4_t wf[2][NB], xf[2][NB];                                                                       \
-        CUBERT_LOAD_FRAGS(CUR, 0, wf[0], xf[0]);                                                            \
-        CUBERT_FENCE_FRAGS(wf[0], xf[0]);                                                                   \
-        _Pragma("unroll") for (int kk = 0; kk < 4; ++kk) {                                                  \
-            if (kk < 3) CUBERT_LOAD_FRAGS(CUR, kk + 1, wf[(kk + 1) & 1], xf[(kk + 1) & 1]);                 \
-            _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                  \
-                _Pragma("unroll") for (int j = 0; j < NB; ++j)                                              \
-                    mfma_chunk<ELT>(wf[kk & 1][i], xf[kk & 1][j], acc[i][j]);                               \
-            if (kk < 3) CUBERT_FENCE_FRAGS(wf[(kk + 1) & 1], xf[(kk + 1) & 1]);                             \
+        if constexpr (NS == 4) {                                                                            \
+            /* One 32 x 32 block per wave: a k-slice is a single MFMA, too short to hide the next     */    \
+            /* slice's fragment read behind it.  All eight reads of the step go out together and each */    \
+            /* MFMA waits for its own pair only (LDS reads return in order).                          */    \
+            u32x4_t wf[4][NB], xf[4][NB];                                                                   \
+            _Pragma("unroll") for (int kk = 0; kk < 4; ++kk) CUBERT_LOAD_FRAGS(CUR, kk, wf[kk], xf[kk]);    \
+            asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(wf[0][0]), "+v"(xf[0][0]));                          \
+            mfma_chunk<ELT>(wf[0][0], xf[0][0], acc[0][0]);                                                 \
+            asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(wf[1][0]), "+v"(xf[1][0]));                          \
+            mfma_chunk<ELT>(wf[1][0], xf[1][0], acc[0][0]);                                                 \
+            asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(wf[2][0]), "+v"(xf[2][0]));                          \
+            mfma_chunk<ELT>(wf[2][0], xf[2][0], acc[0][0]);                                                 \
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wf[3][0]), "+v"(xf[3][0]));                          \
+            mfma_chunk<ELT>(wf[3][0], xf[3][0], acc[0][0]);                                                 \
+        } else {                                                                                            \
+            u32x4_t wf[2][NB], xf[2][NB];                                                                   \
+            CUBERT_LOAD_FRAGS(CUR, 0, wf[0], xf[0]);                                                        \
+            CUBERT_FENCE_FRAGS(wf[0], xf[0]);                                                               \
+            _Pragma("unroll") for (int kk = 0; kk < 4; ++kk) {                                              \
+                if (kk < 3) CUBERT_LOAD_FRAGS(CUR, kk + 1, wf[(kk + 1) & 1], xf[(kk + 1) & 1]);             \
+                _Pragma("unroll") for (int i = 0; i < NB; ++i)                                              \
+                    _Pragma("unroll") for (int j = 0; j < NB; ++j)                                          \
+                        mfma_chunk<ELT>(wf[kk & 1][i], xf[kk & 1][j], acc[i][j]);                           \
+                if (kk < 3) CUBERT_FENCE_FRAGS(wf[(kk + 1) & 1], xf[(kk + 1) & 1]);                         \
+            }                                                                                               \
         }                                                                                                   \
         __builtin_amdgcn_sched_barrier(0);  /* nothing moves across the end of the step */                  \
         __builtin_amdgcn_s_waitcnt(WAIT_IMM); /* my share of the next step's tile has landed */            \
