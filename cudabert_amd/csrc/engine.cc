@@ -478,7 +478,8 @@ bool Model::enqueue(int B, int S, bool has_mask) {
 }
 
 // The launch sequence for sequences [b0, b0 + B) (cuda_bert/utils/bert.cu:129-252):
-// 1 + 7 * layers + 1 kernels, no host synchronisation.  `r0` is the first row of
+// 1 + 7 * layers + 1 kernels (1 + 5 * layers + 1 when the GEMMs before the LayerNorms normalise in their
+// epilogue), no host synchronisation.  `r0` is the first row of
 // this part in the internal activation buffers (a multiple of 256, so that a
 // packed operand starts on a block boundary); inputs and the sequence output
 // are indexed by token.
