@@ -277,6 +277,34 @@ def test_split_batch_two_streams_is_bit_identical(pb, tiny_dir, precision, monke
             pb.unload_model(m)
 
 
+def test_v_layout_switch_is_bit_identical(pb, tiny_dir, monkeypatch):
+    """bf16: V kept head-major and transposed by the attention kernel's LDS reads (the default) against
+    V stored transposed by the QKV GEMM: the same bits, padded and unpadded, and within tolerance of
+    the oracle."""
+    wdir = str(tiny_dir / "bf16")
+    npy = W.load_npy_dir(wdir)
+    B, S = 4, 61
+    ids, seg, mask = synth.make_inputs(B, S, [61, 9, 33, 40], vocab=W.TINY.vocab, seed=5, prune=False)
+    outs = []
+    for flag in ("1", "0"):
+        monkeypatch.setenv("CUBERT_V_ROWMAJOR", flag)
+        for varlen in ("0", "1"):
+            monkeypatch.setenv("CUBERT_VARLEN", varlen)
+            m = load(pb, W.TINY, wdir, BF16, B, S)
+            try:
+                pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+            finally:
+                pb.unload_model(m)
+            outs.append((flag, varlen, pooled, seq))
+    seq_ref, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+    valid = mask.astype(bool)
+    assert np.abs(outs[0][3] - seq_ref)[valid].max() < TOL[BF16]
+    assert np.abs(outs[0][2] - pooled_ref).max() < TOL[BF16]
+    for flag, varlen, pooled, seq in outs[1:]:
+        assert np.array_equal(pooled, outs[0][2]), (flag, varlen)
+        assert np.array_equal(seq[valid], outs[0][3][valid]), (flag, varlen)
+
+
 @pytest.mark.parametrize("precision", [F32, BF16])
 @pytest.mark.parametrize("split", ["0", "1"])
 def test_unpadded_pass_matches_padded_on_valid_positions(pb, tiny_dir, precision, split, monkeypatch):
