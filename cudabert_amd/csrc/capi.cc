@@ -53,7 +53,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.precision = cfg.precision;
     opt.graph_max_tokens = cfg.graph_max_tokens;
     opt.graph_cache = env_int("CUBERT_GRAPH_CACHE", 64);
-    opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 8192);
+    opt.split_min_tokens = env_int("CUBERT_SPLIT_MIN_TOKENS", 14336);
     opt.split_parts = env_int("CUBERT_SPLIT_PARTS", 2);
     opt.varlen = env_int("CUBERT_VARLEN", -1);
     opt.split_k = env_int("CUBERT_SPLIT_K", 1) != 0;

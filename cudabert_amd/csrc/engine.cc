@@ -315,7 +315,8 @@ bool Model::run_compact(const int* lens, int B, int S) {
     B_ = B;
     S_ = S;
     last_compact_ = true;
-    const long tokens = (long)B * S;
+    long tokens = 0;                  // rows this pass computes: the valid tokens
+    for (int b = 0; b < B; ++b) tokens += lens[b];
     int parts = opt_.split_parts < kMaxParts ? opt_.split_parts : kMaxParts;
     if (parts > B) parts = B;
     if (parts < 1 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens) parts = 1;
