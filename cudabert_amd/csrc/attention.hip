@@ -70,7 +70,19 @@ __global__ __launch_bounds__(256) void attention_kernel(
         for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
     float run_max = -INFINITY, run_sum = 0.0f;
 
+    // Key blocks in which every key is masked are skipped: with at least one visible key in the row
+    // their probabilities are exactly zero in float32 (exp of less than -9000), whether they are met
+    // before or after a visible block (the rescaling by exp(-9000) = 0 wipes what they added), so the
+    // result has the bits of walking them.  If no key at all is visible nothing is skipped.
+    unsigned long long live = 0ull;
+    for (int blk = 0; blk * 32 < S && blk < 64; ++blk) {
+        const float m = lane < 32 ? mrow[blk * 32 + lane] : -INFINITY;       // mrow has Sp entries
+        if (__ballot(m > -5000.0f) != 0ull) live |= 1ull << blk;
+    }
+    if (live == 0ull || S > 64 * 32) live = ~0ull;
+
     for (int k0 = 0; k0 < S; k0 += 32) {
+        if (!((live >> ((k0 >> 5) & 63)) & 1ull)) continue;
         // ---- scores^T block: rows = keys k0..k0+31, column = my query ----
         int krow = k0 + l32;
         krow = krow < S ? krow : S - 1;
