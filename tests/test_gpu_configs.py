@@ -390,3 +390,36 @@ def test_reference_benchmark_entry_point_runs(pb, base_ckpt, tmp_path, monkeypat
     ids, seg, mask = pb.seed_batch(2, 32)
     _, pooled_ref = O.forward_torch(base_ckpt.npy_raw, W.BASE.heads, ids, seg, mask)
     assert err(np.array(vals), pooled_ref[0, :10]) < TOL[F32]
+
+
+# ------------------------------------------------------- odd shapes through every path ----
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,S", [(90, 161), (70, 100), (128, 60), (33, 199)])
+def test_odd_shapes_reach_every_path_against_the_oracle(pb, tmp_path, monkeypatch, B, S):
+    """A two-layer model of BERT-base width on batch shapes that are no multiple of any tile: 14 490
+    token rows (two streams, LayerNorm in the GEMM epilogue), 7 000 and 7 680 (one stream, fused
+    LayerNorm), 6 567 (about 5 400 valid rows: separate LayerNorm kernels in the unpadded pass); ragged
+    lengths, one mask with holes; padded and unpadded pass against the float32 oracle, bf16."""
+    import dataclasses
+    dims = dataclasses.replace(W.BASE, layers=2, vocab=2000, max_pos=512)
+    state = W.bf16_representable(W.synth_state(dims, seed=11, degenerate=False))
+    W.export_npy_dir(state, str(tmp_path))
+    npy = W.load_npy_dir(str(tmp_path))
+    rng = np.random.default_rng(B * 1000 + S)
+    lens = rng.integers((2 * S) // 3, S + 1, size=B)
+    lens[0] = S
+    ids, seg, mask = synth.make_inputs(B, S, lens, vocab=dims.vocab, seed=S, prune=False)
+    if B % 2 == 0:
+        mask[1, 2:5] = 0                       # not a prefix: the unpadded pass must decline and run padded
+    seq_ref, pooled_ref = O.forward_torch(npy, dims.heads, ids, seg, mask)
+    valid = mask.astype(bool)
+    for varlen in ("0", "1"):
+        monkeypatch.setenv("CUBERT_VARLEN", varlen)
+        m = load(pb, dims, str(tmp_path), BF16, B, S)
+        try:
+            pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+        finally:
+            pb.unload_model(m)
+        assert np.isfinite(seq).all()
+        assert np.abs(seq - seq_ref)[valid].max() < TOL[BF16], (varlen, np.abs(seq - seq_ref)[valid].max())
+        assert np.abs(pooled - pooled_ref).max() < TOL[BF16], varlen
