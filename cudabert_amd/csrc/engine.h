@@ -25,7 +25,8 @@ struct ModelOptions {
     int max_batch = 0;         // (0, 0): default capacity of 200*512 tokens
     int max_seq = 0;
     int split_parts = 2;           // number of parts (1..4) a large batch is cut into
-    int split_min_tokens = 14336;  // passes over at least this many token rows run as two halves on two streams (0: never)
+    int split_min_tokens = 14336;  // passes over at least this many token rows run as two halves on two streams (0: never);
+                                   // the C API's default follows the precision
     bool fuse_residual = true;     // residual add in the epilogue of the GEMM before each LayerNorm
     bool fuse_layernorm = true;    // ... and the LayerNorm itself, where the GEMM kernel supports it (bf16, large batches)
     bool v_rowmajor = true;        // bf16, S <= 512: V is stored [B, heads, S, 64] like K; attention transposes on its LDS reads
