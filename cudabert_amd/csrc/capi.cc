@@ -200,6 +200,12 @@ void* cubert_stream(void* model) { return model ? static_cast<void*>(static_cast
 int cubert_hidden_size(void* model) { return model ? static_cast<Model*>(model)->dims().hidden : 0; }
 int cubert_num_classes(void* model) { return model ? static_cast<Model*>(model)->num_classes() : 0; }
 int cubert_precision(void* model) { return model ? static_cast<Model*>(model)->precision() : -1; }
+int cubert_ln_fallbacks(void* model) { return model ? static_cast<Model*>(model)->ln_fallbacks() : 0; }
+int cubert_debug_force_ln_timeout(void* model) {
+    cubert::set_error("");
+    Model* m = as_model(model, "cubert_debug_force_ln_timeout");
+    return (m && m->force_ln_timeout()) ? 0 : 1;
+}
 int cubert_graphs_cached(void* model) { return model ? static_cast<Model*>(model)->graphs_cached() : 0; }
 long cubert_capacity_tokens(void* model) { return model ? static_cast<Model*>(model)->capacity_tokens() : 0; }
 

@@ -58,12 +58,16 @@ __host__ __device__ inline size_t packed_offset(int r, int kbyte, int KB) {
 
 // ---- LayerNorm statistics -------------------------------------------------
 // Every LayerNorm of the engine (the row kernels and the GEMM epilogue that normalises) forms its
-// row statistics the same way, so that a row gets the same bits whichever kernel handles it:
-// the row is cut into slots of 128 features; in a slot 32 lanes hold four consecutive features each,
-// add them as (a + b) + (c + d) (squares likewise) and combine with ln_half_wave_sum; the slot sums are
-// added in slot order starting from zero; ln_finalize turns the totals into mean and 1 / sigma
-// (biased variance as E[x^2] - mean^2, eps 1e-12 inside the square root: cuda_bert/ops/layernorm.cu:
-// 127,167; modeling.py:168-172).
+// row statistics the same way, so that a row gets the same bits whichever kernel handles it.
+// The row is cut into slots of 128 features; in a slot 32 lanes hold four consecutive features each.
+// Per slot (ln_slot_stats): the sum, (a + b) + (c + d) per lane combined by ln_half_wave_sum, and M2, the
+// sum of squared distances from the slot's own mean, taken the same way.  ln_row_mean adds the slot sums
+// in slot order starting from zero; ln_merge_slot adds, again in slot order, M2_s + n_s (mean_s - mean)^2
+// (the pairwise update of Chan et al. for a known total mean); ln_finalize turns the total into
+// 1 / sigma (biased variance, eps 1e-12 inside the square root: modeling.py:168-172).  No difference of
+// large squares is formed anywhere, so a row whose mean is many sigma away from zero keeps its
+// precision, as with the running (Welford) statistics of cuda_bert/ops/layernorm.cu:27-67, 100-135.
+// The helpers spell out their fused multiply-adds so that every caller compiles to the same arithmetic.
 #if defined(__HIPCC__)
 template <int CTRL>
 __device__ __forceinline__ float ln_dpp_lanes(float v) {
@@ -80,15 +84,38 @@ __device__ __forceinline__ float ln_half_wave_sum(float v) {
     return v;
 }
 __device__ __forceinline__ float ln_sum4(float a, float b, float c, float d) { return (a + b) + (c + d); }
-__device__ __forceinline__ float ln_sumsq4(float a, float b, float c, float d) { return (a * a + b * b) + (c * c + d * d); }
-__device__ __forceinline__ void ln_finalize(float sum, float sumsq, float inv_n, float* mean, float* rstd) {
-    const float m = sum * inv_n;
-    const float var = fmaxf(sumsq * inv_n - m * m, 0.0f);
-    *mean = m;
-    *rstd = 1.0f / sqrtf(var + 1e-12f);
+__device__ __forceinline__ float ln_sumsq4(float a, float b, float c, float d) {
+#pragma clang fp contract(off)
+    return __builtin_fmaf(a, a, b * b) + __builtin_fmaf(c, c, d * d);
+}
+// Statistics of one slot.  (a, b, c, d): this lane's four features, zeros if the lane lies past the end of
+// the row (`in` false); inv_count = 1 / (features of the row inside this slot), 1 / 128 for a full slot.
+__device__ __forceinline__ void ln_slot_stats(float a, float b, float c, float d, bool in, float inv_count, float* sum,
+                                              float* m2) {
+#pragma clang fp contract(off)
+    const float s = ln_half_wave_sum(ln_sum4(a, b, c, d));
+    const float mu = s * inv_count;
+    const float da = in ? a - mu : 0.0f, db = in ? b - mu : 0.0f, dc = in ? c - mu : 0.0f, dd = in ? d - mu : 0.0f;
+    *sum = s;
+    *m2 = ln_half_wave_sum(ln_sumsq4(da, db, dc, dd));
+}
+__device__ __forceinline__ float ln_row_mean(float sum_of_slot_sums, float inv_n) {
+#pragma clang fp contract(off)
+    return sum_of_slot_sums * inv_n;
+}
+// m2 + (M2 of a slot about the row mean); count = features in the slot (0: the slot lies past the row).
+__device__ __forceinline__ float ln_merge_slot(float m2, float slot_sum, float slot_m2, float count, float inv_count, float mean) {
+#pragma clang fp contract(off)
+    const float dm = slot_sum * inv_count - mean;
+    return m2 + __builtin_fmaf(count * dm, dm, slot_m2);
+}
+__device__ __forceinline__ float ln_finalize(float m2, float inv_n) {
+#pragma clang fp contract(off)
+    return 1.0f / sqrtf(m2 * inv_n + 1e-12f);
 }
 __device__ __forceinline__ float ln_apply(float x, float mean, float rstd, float gamma, float beta) {
-    return gamma * ((x - mean) * rstd) + beta;
+#pragma clang fp contract(off)
+    return __builtin_fmaf(gamma, (x - mean) * rstd, beta);
 }
 #endif
 

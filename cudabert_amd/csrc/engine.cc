@@ -90,7 +90,8 @@ bool Model::init(const ModelOptions& opt_in) {
         return false;
     }
     CUBERT_HIP_OK(hipSetDevice(opt_.gpu));
-    if (!noalloc_setup_current_device()) return false;
+    // best effort: the allocation-free GEMM entry point looks its scratch address up itself if this did not work
+    if (!noalloc_setup_current_device()) set_error("");
     CUBERT_HIP_OK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
     for (int i = 1; i < kMaxParts; ++i) {
         CUBERT_HIP_OK(hipStreamCreateWithFlags(&side_[i], hipStreamNonBlocking));
@@ -228,6 +229,13 @@ bool Model::init(const ModelOptions& opt_in) {
     return true;
 }
 
+bool Model::force_ln_timeout() {
+    CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    for (int i = 0; i < kMaxParts; ++i)
+        if (!gemm_ln_workspace_force_expiry(ln_ws_ + (size_t)i * ln_ws_bytes_)) return false;
+    return true;
+}
+
 bool Model::check_shape(int B, int S) {
     // Limits inherited from the reference: B*S within the allocated capacity
     // (cuda_bert/utils/manager.cu:100-108), B <= 1024 (ops/batch_matmul.cu:60),
@@ -315,6 +323,8 @@ bool Model::run_compact(const int* lens, int B, int S) {
     B_ = B;
     S_ = S;
     last_compact_ = true;
+    last_classified_ = false;
+    if (lens != last_lens_.data()) last_lens_.assign(lens, lens + B);
     long tokens = 0;                  // rows this pass computes: the valid tokens
     for (int b = 0; b < B; ++b) tokens += lens[b];
     int parts = opt_.split_parts < kMaxParts ? opt_.split_parts : kMaxParts;
@@ -381,6 +391,8 @@ bool Model::run(int B, int S, bool has_mask) {
     B_ = B;
     S_ = S;
     last_compact_ = false;
+    last_has_mask_ = has_mask;
+    last_classified_ = false;
     const long tokens = (long)B * S;
     if (opt_.graph_max_tokens <= 0 || tokens > opt_.graph_max_tokens) return enqueue(B, S, has_mask);
     // One entry per (B, S, mask) shape; the key is injective for every B <= 1024 and any S.
@@ -389,6 +401,7 @@ bool Model::run(int B, int S, bool has_mask) {
     if (it != graphs_.end() && it->second.exec) {
         it->second.last_use = ++graph_clock_;
         CUBERT_HIP_OK(hipGraphLaunch(it->second.exec, stream_));
+        ln_used_ = std::max(ln_used_, it->second.ln_parts);      // sync() looks at the error words of a replayed pass too
         return true;
     }
     if (it == graphs_.end()) {
@@ -403,7 +416,11 @@ bool Model::run(int B, int S, bool has_mask) {
     GraphEntry& ge = graphs_[key];
     hipGraph_t graph = nullptr;
     CUBERT_HIP_OK(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal));
+    const int ln_before = ln_used_;
+    ln_used_ = 0;
     const bool ok = enqueue(B, S, has_mask);
+    ge.ln_parts = ln_used_;
+    ln_used_ = std::max(ln_before, ge.ln_parts);
     const std::string keep = ok ? std::string() : std::string(get_error());
     const hipError_t e = hipStreamEndCapture(stream_, &graph);
     if (!ok) { if (graph) (void)hipGraphDestroy(graph); set_error(keep); return false; }
@@ -598,6 +615,8 @@ bool Model::profile_device(const int* d_ids, const int* d_seg, const int* d_mask
     B_ = B;
     S_ = S;
     last_compact_ = false;
+    last_has_mask_ = d_mask != nullptr;
+    last_classified_ = false;
     profiling_ = true;
     prof_used_ = 0;
     prof_phase_.clear();
@@ -618,45 +637,80 @@ bool Model::profile_device(const int* d_ids, const int* d_seg, const int* d_mask
 bool Model::classify() {
     if (!num_classes_) { set_error("the weight directory holds no classifier_kernel / classifier_bias"); return false; }
     if (B_ <= 0) { set_error("classify() needs a preceding forward pass"); return false; }
+    last_classified_ = true;
     return launch_classifier(pooled_, w_cls_, b_cls_, cls_, B_, opt_.dims.hidden, num_classes_, stream_);
+}
+
+// The last pass once more, launch by launch, from the inputs (and, for an unpadded pass, the lengths) it left behind.
+bool Model::rerun_last() {
+    const bool classified = last_classified_;
+    bool ok;
+    if (last_compact_) {
+        ok = run_compact(last_lens_.data(), B_, S_);
+    } else {
+        last_classified_ = false;
+        ok = enqueue(B_, S_, last_has_mask_);
+    }
+    return ok && (!classified || classify());
 }
 
 bool Model::sync() {
     CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+    recovered_ = false;
     if (ln_used_ > 0) {
         // A workgroup of a GEMM that normalises in its epilogue gives up after a bounded wait for its
         // partners and raises word 0 of its workspace; the results of that pass are then not valid.
+        // Every used part is looked at (and put back to zero) before anything else happens.
         const int parts = ln_used_;
         ln_used_ = 0;
+        bool raised = false;
         for (int i = 0; i < parts; ++i) {
             int flag = 0;
             CUBERT_HIP_OK(hipMemcpy(&flag, ln_ws_ + (size_t)i * ln_ws_bytes_, sizeof(int), hipMemcpyDeviceToHost));
             if (flag != 0) {
                 CUBERT_HIP_OK(hipMemset(ln_ws_ + (size_t)i * ln_ws_bytes_, 0, ln_ws_bytes_));
-                set_error("a GEMM with the LayerNorm in its epilogue timed out waiting for the workgroups it shares rows with");
-                return false;
+                raised = true;
             }
         }
+        if (raised) {
+            // Nothing is lost: the inputs of the pass are still on the device.  The pass is repeated with the
+            // LayerNorms as kernels of their own (which wait for nobody), this model keeps them that way, and
+            // the graphs captured with the fused kernels go.
+            opt_.fuse_layernorm = false;
+            ++ln_fallbacks_;
+            if (!evict_graphs(0)) return false;
+            graphs_.clear();
+            if (!rerun_last()) return false;
+            CUBERT_HIP_OK(hipStreamSynchronize(stream_));
+            recovered_ = true;
+        }
+    }
+    return true;
+}
+
+bool Model::copy_out(float* out, const float* dev, size_t floats) {
+    CUBERT_HIP_OK(hipMemcpyAsync(out, dev, floats * 4, hipMemcpyDeviceToHost, stream_));
+    if (!sync()) return false;
+    if (recovered_) {       // the copy above ran before the pass was repeated
+        CUBERT_HIP_OK(hipMemcpyAsync(out, dev, floats * 4, hipMemcpyDeviceToHost, stream_));
+        CUBERT_HIP_OK(hipStreamSynchronize(stream_));
     }
     return true;
 }
 
 bool Model::copy_pooled(float* out) {
     if (!out || B_ <= 0) { set_error("no result to copy"); return false; }
-    CUBERT_HIP_OK(hipMemcpyAsync(out, pooled_, (size_t)B_ * opt_.dims.hidden * 4, hipMemcpyDeviceToHost, stream_));
-    return sync();
+    return copy_out(out, pooled_, (size_t)B_ * opt_.dims.hidden);
 }
 
 bool Model::copy_seq(float* out) {
     if (!out || B_ <= 0) { set_error("no result to copy"); return false; }
-    CUBERT_HIP_OK(hipMemcpyAsync(out, seq_ptr(), (size_t)B_ * S_ * opt_.dims.hidden * 4, hipMemcpyDeviceToHost, stream_));
-    return sync();
+    return copy_out(out, seq_ptr(), (size_t)B_ * S_ * opt_.dims.hidden);
 }
 
 bool Model::copy_cls(float* out) {
     if (!out || B_ <= 0 || !num_classes_) { set_error("no result to copy"); return false; }
-    CUBERT_HIP_OK(hipMemcpyAsync(out, cls_, (size_t)B_ * num_classes_ * 4, hipMemcpyDeviceToHost, stream_));
-    return sync();
+    return copy_out(out, cls_, (size_t)B_ * num_classes_);
 }
 
 }  // namespace cubert

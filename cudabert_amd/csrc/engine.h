@@ -67,6 +67,7 @@ class Model {
                  kNumPhases };
     bool profile_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S, float* phase_ms);
     bool sync();
+    bool copy_out(float* host_out, const float* dev, size_t floats);   // D2H + sync (again after a repeated pass)
     bool copy_pooled(float* host_out);                 // D2H + sync, B*hidden floats
     bool copy_seq(float* host_out);                    // D2H + sync, B*S*hidden floats
     bool copy_cls(float* host_out);                    // D2H + sync, B*num_classes floats
@@ -82,6 +83,8 @@ class Model {
     int last_batch() const { return B_; }
     int last_seq() const { return S_; }
     int graphs_cached() const;                         // instantiated hipGraphs held
+    int ln_fallbacks() const { return ln_fallbacks_; } // passes repeated with separate LayerNorm kernels (see sync())
+    bool force_ln_timeout();                           // test aid: the next pass with a LayerNorm epilogue times out
     size_t weight_bytes() const { return weight_bytes_; }
     size_t activation_bytes() const { return act_bytes_; }
 
@@ -93,6 +96,7 @@ class Model {
     bool enqueue(int B, int S, bool has_mask);         // the launch sequence (one or two parts)
     bool enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mask, hipStream_t st, const Compact* cp = nullptr);
     bool run_compact(const int* h_lens, int B, int S);
+    bool rerun_last();                                 // the last pass once more, eagerly, from the inputs still on the device
     bool mark(int phase);                              // profiling: event before a launch
 
     ModelOptions opt_;
@@ -131,13 +135,21 @@ class Model {
     unsigned char* ln_ws_ = nullptr;   // kMaxParts workspaces of the GEMMs that normalise in their epilogue
     size_t ln_ws_bytes_ = 0;           // size of one of them
     int ln_used_ = 0;                  // parts whose workspaces such GEMMs used since sync() last looked at their error words
+    int ln_fallbacks_ = 0;             // times sync() found an error word raised and repeated the pass without the fused LayerNorm
+    bool recovered_ = false;           // the last sync() repeated the pass: copies enqueued before it carry the discarded results
+    bool last_has_mask_ = false, last_classified_ = false;
+    std::vector<int> last_lens_;       // lengths of the last unpadded pass
     bool last_compact_ = false;
     int cur_parts_ = 1;          // parts of the pass being enqueued
     int B_ = 0, S_ = 0;
     // hipGraph cache: one entry per (B, S, mask) shape, captured on second sight, at most
     // opt_.graph_cache instantiated at a time (least recently used goes first).
     int max_graphs() const { return opt_.graph_cache > 0 ? opt_.graph_cache : 1; }
-    struct GraphEntry { hipGraphExec_t exec = nullptr; unsigned long long last_use = 0; };
+    struct GraphEntry {
+        hipGraphExec_t exec = nullptr;
+        unsigned long long last_use = 0;
+        int ln_parts = 0;        // parts whose LayerNorm-epilogue workspaces the captured pass uses
+    };
     std::map<unsigned long long, GraphEntry> graphs_;
     unsigned long long graph_clock_ = 0;
     bool evict_graphs(int keep);

@@ -295,7 +295,7 @@ bool launch_epi(const GemmDev& d, int epi, int bt, hipStream_t stream) {
 
 namespace {
 // Workspace of the LayerNorm epilogue: flag words, two counters per band of rows (a fixed number of
-// bands, so that launches with different M agree on where the counters are), then (sum, sum of squares)
+// bands, so that launches with different M agree on where the counters are), then (sum, M2 about the slot mean)
 // for every row and every 128-feature slot (at most 8).
 constexpr size_t kLnMaxBands = 16384;
 size_t ln_stats_offset() { return ((gemm_detail::kLnCntFirst + 2 * kLnMaxBands) * sizeof(int) + 255) / 256 * 256; }
@@ -306,6 +306,15 @@ size_t gemm_ln_workspace_bytes(size_t M) { return ln_stats_offset() + ((M + 255)
 namespace {
 bool ln_shape_ok(int N, int K, int elt) { return elt == kBF16 && N > 0 && N % 256 == 0 && N <= 1024 && K % 32 == 0 && K >= 64; }
 }  // namespace
+
+bool gemm_ln_workspace_force_expiry(void* ln_ws) {
+    if (!ln_ws) { set_error("gemm: null workspace"); return false; }
+    const int limit = 1, stuck = -1000000;
+    int* w = static_cast<int*>(ln_ws);
+    CUBERT_HIP_OK(hipMemcpy(w + 1, &limit, sizeof(int), hipMemcpyHostToDevice));
+    CUBERT_HIP_OK(hipMemcpy(w + gemm_detail::kLnCntFirst, &stuck, sizeof(int), hipMemcpyHostToDevice));
+    return true;
+}
 
 // Tile of a GEMM with the LayerNorm in its epilogue, 0 if the separate kernels are the better choice.
 // Measured on MI355X (N = 768 and 1024, K = N and 4 N): from about 6000 rows on the fused kernel beats

@@ -36,7 +36,7 @@ struct GemmDev {
     unsigned char* ln_xb;                 // bf16 copy of the result (may be null)
     int ln_xb_packed;
     int* ln_cnt;                          // [0] error flag, [1] poll limit (0: default), [kLnCntFirst + band] arrivals, [.. + ln_bands + band] departures
-    unsigned long long* ln_stats;         // [row][2 * tiles_n] (sum, sum of squares) as two floats in 64 bits
+    unsigned long long* ln_stats;         // [row][2 * tiles_n] (sum, M2 about the slot's mean) as two floats in 64 bits
     int ln_bands;
 };
 
@@ -332,7 +332,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
 // N = 256 * tiles_n features, float32 row-major, plus an optional bf16 copy (the next GEMM's operand).
 //
 // A workgroup holds 256 of a row's features, so the tiles_n workgroups of one band of rows have to
-// agree on the row statistics.  Every wave (128 features of its rows) publishes (sum, sum of squares)
+// agree on the row statistics.  Every wave (128 features of its rows) publishes (sum, M2 about its own mean)
 // per row in device memory, the workgroup counts itself in on the band's arrival counter, waits until
 // all tiles_n workgroups have, and reads the 2 * tiles_n partial sums of its rows.  The accumulators go
 // through the wave's LDS staging once (whole row segments come out, bias and residual are added to
@@ -422,8 +422,8 @@ __device__ __forceinline__ void gemm_epilogue_ln(const GemmDev& p, f32x16_t (&ac
         const f32x4_t bias4 = *reinterpret_cast<const f32x4_t*>(p.bias + n);
         ln_stream_rows<NBI, NBJ, 4>(acc, buf, l32, g, rrow, rc, bias4, r_rsrc, (m_base + rrow) * row_bytes + n * 4, row_bytes,
                                  [&](int j, int s, const f32x4_t& d) {
-            const float t = ln_half_wave_sum(ln_sum4(d[0], d[1], d[2], d[3]));
-            const float q = ln_half_wave_sum(ln_sumsq4(d[0], d[1], d[2], d[3]));
+            float t, q;                                       // the slot's sum and M2 about the slot's mean
+            ln_slot_stats(d[0], d[1], d[2], d[3], true, 0.0078125f, &t, &q);
             const int pair = j * NIT + s;                     // compile-time after unrolling
             if (rc == (pair & 31)) { ksum[pair >> 5] = t; ksq[pair >> 5] = q; }
             // The sums stay in the registers of the accumulators they were made from (block column j
@@ -497,18 +497,25 @@ __device__ __forceinline__ void gemm_epilogue_ln(const GemmDev& p, f32x16_t (&ac
         for (int t = 0; t < NP; ++t) {
             const int pair = t * 32 + rc;
             const int rl = 32 * (pair / NIT) + RPI * (pair % NIT) + rrow;     // row within the wave's rows
-            float sum = 0.0f, sq = 0.0f;
+            float sum = 0.0f;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 if (2 * c < slots) {          // a wave-uniform branch; slots is even
-                    sum += raw[t][c][0]; sq += raw[t][c][1];
-                    sum += raw[t][c][2]; sq += raw[t][c][3];
+                    sum += raw[t][c][0];
+                    sum += raw[t][c][2];
                 }
             }
-            float mean, rstd;
-            ln_finalize(sum, sq, invn, &mean, &rstd);
+            const float mean = ln_row_mean(sum, invn);
+            float m2 = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (2 * c < slots) {
+                    m2 = ln_merge_slot(m2, raw[t][c][0], raw[t][c][1], 128.0f, 0.0078125f, mean);
+                    m2 = ln_merge_slot(m2, raw[t][c][2], raw[t][c][3], 128.0f, 0.0078125f, mean);
+                }
+            }
             statbuf[2 * rl] = mean;
-            statbuf[2 * rl + 1] = rstd;
+            statbuf[2 * rl + 1] = ln_finalize(m2, invn);
         }
     }
     __syncthreads();                                       // every wave holds its statistics: the band can be left

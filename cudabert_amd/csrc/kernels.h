@@ -85,6 +85,10 @@ struct GemmParams {
 bool launch_gemm(const GemmParams& p, hipStream_t stream);
 // Workspace of a GEMM with the LayerNorm in its epilogue (GemmParams::ln_ws) for up to M rows.
 size_t gemm_ln_workspace_bytes(size_t M);
+// Test aid: puts a workspace into a state in which the workgroups of row band 0 can never see their band complete
+// (arrival counter far below zero) and give up after a single poll, so that the bounded wait expires -- every kernel
+// still runs to its end -- and the error word gets raised.  Synchronous.
+bool gemm_ln_workspace_force_expiry(void* ln_ws);
 // True if launch_gemm can run the LayerNorm of a [M, N] float32 result in the epilogue of a
 // bf16 GEMM with reduction length K.
 bool gemm_ln_supported(int M, int N, int K, int elt);

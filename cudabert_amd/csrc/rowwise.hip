@@ -33,23 +33,39 @@ __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H
                                                 const float* __restrict__ beta, float* xrow,
                                                 bf16_t* xb, int row, int xb_packed) {
     // Row statistics in the engine's canonical order (common.h): chunk c holds the slots 2 c (lanes
-    // 0..31) and 2 c + 1 (lanes 32..63); slots past the row's end contribute zero.
-    float sum = 0.0f, sumsq = 0.0f;
+    // 0..31) and 2 c + 1 (lanes 32..63); slots past the row's end hold no features and add nothing.
+    const bool upper = lane >= 32;
+    float ssum[2 * kMaxChunks], sm2[2 * kMaxChunks], scnt[2 * kMaxChunks], sinv[2 * kMaxChunks];
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int left = H - 128 * (2 * c + u);
+            const int cnt = left < 0 ? 0 : (left > 128 ? 128 : left);
+            scnt[2 * c + u] = (float)cnt;
+            sinv[2 * c + u] = cnt > 0 ? 1.0f / (float)cnt : 0.0f;
+        }
         const bool in = c * 256 + lane * 4 < H;
-        const float t = ln_half_wave_sum(in ? ln_sum4(v[c][0], v[c][1], v[c][2], v[c][3]) : 0.0f);
-        const float q = ln_half_wave_sum(in ? ln_sumsq4(v[c][0], v[c][1], v[c][2], v[c][3]) : 0.0f);
-        // every lane gets the lower slot's sum first, then the upper one's
+        float t, q;
+        ln_slot_stats(in ? v[c][0] : 0.0f, in ? v[c][1] : 0.0f, in ? v[c][2] : 0.0f, in ? v[c][3] : 0.0f, in,
+                      upper ? sinv[2 * c + 1] : sinv[2 * c], &t, &q);
+        // every lane gets both slots' statistics
         const float t_other = __shfl_xor(t, 32), q_other = __shfl_xor(q, 32);
-        const bool upper = lane >= 32;
-        sum += upper ? t_other : t;
-        sumsq += upper ? q_other : q;
-        sum += upper ? t : t_other;
-        sumsq += upper ? q : q_other;
+        ssum[2 * c] = upper ? t_other : t;
+        sm2[2 * c] = upper ? q_other : q;
+        ssum[2 * c + 1] = upper ? t : t_other;
+        sm2[2 * c + 1] = upper ? q : q_other;
     }
-    float mean, rstd;
-    ln_finalize(sum, sumsq, 1.0f / (float)H, &mean, &rstd);
+    const float inv_n = 1.0f / (float)H;
+    float sum = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 2 * kMaxChunks; ++s) sum += ssum[s];
+    const float mean = ln_row_mean(sum, inv_n);
+    float m2 = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 2 * kMaxChunks; ++s)
+        if (128 * s < H) m2 = ln_merge_slot(m2, ssum[s], sm2[s], scnt[s], sinv[s], mean);
+    const float rstd = ln_finalize(m2, inv_n);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
         const int i = c * 256 + lane * 4;

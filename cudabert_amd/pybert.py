@@ -90,7 +90,8 @@ lib.cubert_pooled_ptr.argtypes = [c_void_p]
 lib.cubert_pooled_ptr.restype = c_void_p
 lib.cubert_stream.argtypes = [c_void_p]
 lib.cubert_stream.restype = c_void_p
-for _n in ("cubert_hidden_size", "cubert_num_classes", "cubert_precision", "cubert_graphs_cached"):
+for _n in ("cubert_hidden_size", "cubert_num_classes", "cubert_precision", "cubert_graphs_cached", "cubert_ln_fallbacks",
+           "cubert_debug_force_ln_timeout"):
     getattr(lib, _n).argtypes = [c_void_p]
     getattr(lib, _n).restype = c_int
 lib.cubert_capacity_tokens.argtypes = [c_void_p]
@@ -199,10 +200,31 @@ SEED_SEGMENTS = [0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1]
 SEED_MASK = [1, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0]
 
 
+def filling_inputs(words, seq_length):
+    """cuda_bert/pybert.py:44-53: stretches a seed row to seq_length by cycling through all but its last entry and
+    keeping the last entry at the end; a row that is already longer comes back unchanged.  Returns a new list."""
+    body, last = list(words[:-1]), words[-1]
+    n = len(body)
+    body.extend(body[i % n] for i in range(n, seq_length - 1))
+    return body + [last]
+
+
+def batch_inputs(input, batchsize):
+    """cuda_bert/pybert.py:55-59: the row repeated batchsize times."""
+    return [input] * batchsize
+
+
+def warp_inputs(indexed_tokens, segments_ids, attention_masks):
+    """cuda_bert/pybert.py:61-65: the three nested lists as int32 arrays."""
+    return tuple(numpy.array(a).astype(numpy.int32) for a in (indexed_tokens, segments_ids, attention_masks))
+
+
 def seed_batch(batchsize, seq_length):
     """The reference benchmarks' input as int32 [batchsize, seq_length] arrays (ids, segments, mask):
     each 11-entry seed row is stretched to seq_length by cycling through its first ten entries and
-    keeping its last entry in the last column, and the row is repeated batchsize times."""
+    keeping its last entry in the last column, and the row is repeated batchsize times.  Equal to
+    warp_inputs(*[batch_inputs(filling_inputs(seed, seq_length), batchsize) for each seed]) from 11 columns on;
+    shorter requests are cut to seq_length here, where filling_inputs returns all 11 entries."""
     if seq_length < 2:
         raise ValueError("seq_length must be at least 2")
     cycle = numpy.arange(seq_length - 1) % 10

@@ -154,6 +154,17 @@ int cubert_hidden_size(void* model);
 int cubert_num_classes(void* model);
 int cubert_precision(void* model);
 int cubert_graphs_cached(void* model);
+/* How often a pass of this model was repeated with the LayerNorms as kernels of their own.  The bf16 GEMMs before the
+ * LayerNorms of large batches normalise in their epilogue: the workgroups that share a row wait for each other, for a
+ * bounded time.  If that wait ever expires (the chip shared with another process in a way that keeps partners from being
+ * resident together), the next synchronising call notices, repeats the pass from the inputs still on the device with
+ * separate LayerNorm kernels -- the results are the same bits -- keeps this model on those kernels, and counts it here.
+ * No reference counterpart: cuda_bert/ops/layernorm.cu:136-206 is always a kernel of its own.
+ * (CUBERT_FUSE_LAYERNORM=0 at init never fuses.) */
+int cubert_ln_fallbacks(void* model);
+/* Test aid for the above: leaves the model's LayerNorm-epilogue workspaces in a state in which the next pass that uses
+ * them cannot see row band 0 complete and gives up after one poll.  Every kernel still runs to its end.  Returns 0. */
+int cubert_debug_force_ln_timeout(void* model);
 long cubert_capacity_tokens(void* model);
 
 /* ---- single kernels on caller-owned device memory (parity tests, roofline

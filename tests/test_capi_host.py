@@ -163,3 +163,23 @@ def test_seed_batch(pb):
     assert ids[0, -1] == pb.SEED_IDS[-1] and seg[0, -1] == 1 and mask[0, -1] == 0
     ids11, _, mask11 = pb.seed_batch(1, 11)
     assert list(ids11[0]) == pb.SEED_IDS and list(mask11[0]) == pb.SEED_MASK
+
+
+def test_reference_input_helpers():
+    """filling_inputs / batch_inputs / warp_inputs of cuda_bert/pybert.py:44-65, which user scripts import from the
+    binding module: the seed row is stretched by cycling through all but its last entry, which stays last."""
+    pb = pytest.importorskip("cudabert_amd.pybert")
+    seed = list(range(100, 111))                       # 11 entries
+    assert pb.filling_inputs(seed, 11) == seed
+    assert pb.filling_inputs(seed, 5) == seed           # shorter requests return the row unchanged
+    got = pb.filling_inputs(seed, 25)
+    assert len(got) == 25 and got[-1] == 110 and got[:10] == seed[:10]
+    assert got[10:24] == [100 + (i % 10) for i in range(10, 24)]
+    assert seed == list(range(100, 111))                # the caller's list is untouched
+    rows = pb.batch_inputs(got, 3)
+    assert len(rows) == 3 and all(r == got for r in rows)
+    a, b, c = pb.warp_inputs(rows, rows, rows)
+    assert a.dtype == np.int32 and a.shape == (3, 25) and np.array_equal(a, b) and np.array_equal(b, c)
+    ids, seg, mask = pb.seed_batch(3, 25)
+    want = pb.warp_inputs(*[pb.batch_inputs(pb.filling_inputs(list(s), 25), 3) for s in (pb.SEED_IDS, pb.SEED_SEGMENTS, pb.SEED_MASK)])
+    assert np.array_equal(ids, want[0]) and np.array_equal(seg, want[1]) and np.array_equal(mask, want[2])

@@ -206,6 +206,61 @@ def test_layernorm_in_gemm_epilogue_inside_a_captured_graph(pb, base_ckpt):
     assert err(first[1][:n], seq_ref) < TOL[BF16] and err(first[0][:n], pooled_ref) < TOL[BF16]
 
 
+def test_layernorm_epilogue_timeout_is_recovered_not_fatal(pb, base_ckpt, monkeypatch):
+    """The workgroups of a GEMM that normalises in its epilogue wait for their partners for a bounded time.  When that
+    wait expires (forced here from the host: band 0 can never complete and the poll limit is one; every kernel still
+    ends normally), the next synchronising call repeats the pass with separate LayerNorm kernels, keeps the model on
+    them and counts it; the caller gets the bits of a model that never fused.  Seen on an eager pass and on the replay
+    of a captured graph (whose launch never passes through the code that enqueues kernels)."""
+    D = W.BASE
+    B, S = 33, 200
+    lens = np.random.default_rng(5).integers(190, S + 1, size=B)       # >= 6144 valid tokens: the unpadded pass fuses too
+    lens[0] = S
+    ids, seg, mask = synth.make_inputs(B, S, list(lens), seed=78)
+    monkeypatch.setenv("CUBERT_FUSE_LAYERNORM", "0")
+    m = load(pb, D, base_ckpt.bf16x, BF16, B, S, graph=0)
+    try:
+        want = pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)
+        assert pb.lib.cubert_ln_fallbacks(m) == 0
+    finally:
+        pb.unload_model(m)
+    monkeypatch.delenv("CUBERT_FUSE_LAYERNORM")
+
+    def same(got):
+        return all(np.array_equal(a, b) for a, b in zip(got, want))
+
+    for graph, warm in ((0, 1), (8192, 3)):        # 3 calls: eager, capture, replay
+        m = load(pb, D, base_ckpt.bf16x, BF16, B, S, graph=graph)
+        try:
+            for _ in range(warm):
+                assert same(pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True))       # fused: the same bits anyway
+            assert pb.lib.cubert_ln_fallbacks(m) == 0 and pb.lib.cubert_graphs_cached(m) == (1 if graph else 0)
+            pb.check(pb.lib.cubert_debug_force_ln_timeout(m))
+            assert same(pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)), graph
+            assert pb.lib.cubert_ln_fallbacks(m) == 1
+            assert pb.lib.cubert_graphs_cached(m) == 0          # graphs with the fused kernels are gone
+            for _ in range(3):                                   # and the model carries on (capturing anew)
+                assert same(pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True))
+            assert pb.lib.cubert_ln_fallbacks(m) == 1
+            # pooled-only host call: takes the unpadded pass, which is repeated the same way
+            out = np.zeros((B, D.hidden), np.float32)
+            pb.bert(m, out, ids, seg, B, S, mask)
+            assert np.array_equal(out, want[0])
+        finally:
+            pb.unload_model(m)
+    # the unpadded pass (two stream parts above 14336 rows; here one) times out and is repeated too
+    monkeypatch.setenv("CUBERT_VARLEN", "1")
+    m = load(pb, D, base_ckpt.bf16x, BF16, B, S, graph=0)
+    try:
+        pb.check(pb.lib.cubert_debug_force_ln_timeout(m))
+        pooled, seq, cls = pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)
+        valid = mask.astype(bool)
+        assert pb.lib.cubert_ln_fallbacks(m) == 1
+        assert np.array_equal(pooled, want[0]) and np.array_equal(cls, want[2]) and np.array_equal(seq[valid], want[1][valid])
+    finally:
+        pb.unload_model(m)
+
+
 # ------------------------------------------------------------------ configuration 4 ----
 
 def test_cfg4_large_b64_s512_skewed(pb, large_ckpt):

@@ -264,11 +264,53 @@ def test_add_layernorm(pb, H, y_elt):
     assert np.array_equal(xb.float().cpu().numpy(), bf16_round(got))     # bf16 copy is the RNE of the f32 result
 
 
-def test_embed_layernorm(pb):
+@pytest.mark.parametrize("H", [320, 768, 1024])
+@pytest.mark.parametrize("offset", [30.0, 100.0])
+@pytest.mark.parametrize("parts", [1, 3])
+def test_add_layernorm_rows_far_from_zero(pb, H, offset, parts):
+    """Rows whose mean lies 30 and 100 standard deviations from zero (either sign): the statistics are
+    formed from deviations (per 128-feature slot, merged by the pairwise update), never as a difference of
+    large squares, so the result keeps float32 precision.  One-pass E[x^2] - mean^2 is off by 6e-4 / 8e-3 here.
+    At 100 sigma the inputs themselves are spaced 7.6e-6 sigma apart and the mean of 1024 of them is known to
+    about 1e-5 sigma, which bounds what any float32 kernel can deliver (tolerance 4e-5 there, 2e-5 at 30)."""
+    rng = np.random.default_rng(int(H + offset))
+    rows = 515
+    sign = np.where(rng.random((rows, 1)) < 0.5, -1.0, 1.0)
+    x = (rng.standard_normal((rows, H)) + offset * sign * 0.75).astype(np.float32)
+    y = (rng.standard_normal((parts, rows, H)) * 0.5 + offset * sign * 0.25 / parts).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(H)).astype(np.float32)
+    s = x.astype(np.float64) + y.astype(np.float64).sum(0)
+    u = s.mean(-1, keepdims=True)
+    var = ((s - u) ** 2).mean(-1, keepdims=True)
+    assert np.abs(u / np.sqrt(var)).min() > 0.7 * offset
+    ref = g * ((s - u) / np.sqrt(var + 1e-12)) + b
+    xd, yd, gd, bd = dev(x), dev(y), dev(g), dev(b)
+    flags = (parts & 0xff) << 8 if parts > 1 else 0
+    pb.check(pb.lib.cubert_op_add_layernorm(xd.data_ptr(), yd.data_ptr(), F32, gd.data_ptr(), bd.data_ptr(), None, rows, H,
+                                            flags, stream()))
+    torch.cuda.synchronize()
+    # the float32 sum x + y that the kernel normalises is itself rounded at this magnitude: compare against the
+    # statistics of what float32 addition in the kernel's order gives
+    s32 = y[0].copy()
+    for p in range(1, parts):
+        s32 = s32 + y[p]
+    s32 = (x + s32).astype(np.float64)
+    u32 = s32.mean(-1, keepdims=True)
+    ref32 = g * ((s32 - u32) / np.sqrt(((s32 - u32) ** 2).mean(-1, keepdims=True) + 1e-12)) + b
+    err = np.abs(xd.cpu().numpy() - ref32).max()
+    assert err < (2e-5 if offset <= 30 else 4e-5), err
+    assert np.abs(xd.cpu().numpy() - ref).max() < 2e-5 * offset          # and the exact sum within its own rounding
+
+
+@pytest.mark.parametrize("offset", [0.0, 30.0, 100.0])
+def test_embed_layernorm(pb, offset):
     rng = np.random.default_rng(11)
     B, S, H, V = 3, 37, 768, 500
     Sp = 64
     word = rng.standard_normal((V, H)).astype(np.float32)
+    # rows far from zero, either sign (see test_add_layernorm_rows_far_from_zero)
+    word += (offset * np.where(rng.random((V, 1)) < 0.5, -1.0, 1.0)).astype(np.float32)
     pos = rng.standard_normal((64, H)).astype(np.float32)
     typ = rng.standard_normal((2, H)).astype(np.float32)
     g = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
@@ -288,7 +330,12 @@ def test_embed_layernorm(pb):
                                               madd.data_ptr(), B, S, H, V, 2, 0, stream()))
     torch.cuda.synchronize()
     got = x.cpu().numpy().reshape(B, S, H)
-    assert np.abs(got - ref).max() < 2e-5
+    # float32 rounding of the three-way sum at the rows' magnitude comes on top of the kernel's own error
+    assert np.abs(got - ref).max() < 2e-5 * max(1.0, offset / 3)
+    e32 = ((word[ids] + pos[np.arange(S)][None]) + typ[seg]).astype(np.float64)
+    u32 = e32.mean(-1, keepdims=True)
+    ref32 = g * ((e32 - u32) / np.sqrt(((e32 - u32) ** 2).mean(-1, keepdims=True) + 1e-12)) + b
+    assert np.abs(got - ref32).max() < (2e-5 if offset <= 30 else 4e-5)
     m = madd.cpu().numpy()
     assert np.array_equal(m[:, :S], (1.0 - mask) * np.float32(-10000.0))
     assert np.isneginf(m[:, S:]).all()
@@ -680,3 +727,41 @@ def test_gemm_with_residual_and_layernorm_in_the_epilogue(pb, M, N, K, tile, pac
     assert pb.lib.cubert_op_gemm_residual_layernorm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Rd.data_ptr(), gd.data_ptr(),
                                                     bed.data_ptr(), buf[1:].data_ptr(), xb.data_ptr(), ws.data_ptr(), M, N - 8, K, K,
                                                     tile, gflags, stream()) != 0
+
+
+@pytest.mark.parametrize("M,N,K,tile", [(1000, 1024, 1024, 256), (777, 768, 256, 384), (6400, 1024, 4096, 0)])
+@pytest.mark.parametrize("offset", [30.0, 100.0])
+def test_layernorm_epilogue_rows_far_from_zero(pb, M, N, K, tile, offset):
+    """The LayerNorm epilogue on rows whose mean lies 30 / 100 standard deviations from zero (either sign), against
+    float64, and bit for bit against the same GEMM followed by the LayerNorm row kernel (one recipe for the
+    statistics, whichever kernel normalises)."""
+    rng = np.random.default_rng(int(M + N + K + offset))
+    X = bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    Wt = bf16_round((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    b = rng.standard_normal(N).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+    be = (0.1 * rng.standard_normal(N)).astype(np.float32)
+    prod = (torch.from_numpy(X).double() @ torch.from_numpy(Wt).double().T).numpy() + b
+    R0 = rng.standard_normal((M, N)) * 2
+    sigma = (prod + R0).std(-1, keepdims=True)
+    R = (R0 + offset * sigma * np.where(rng.random((M, 1)) < 0.5, -1.0, 1.0)).astype(np.float32)
+    pre = prod + R
+    assert np.abs(pre.mean(-1) / pre.std(-1)).min() > 0.9 * offset
+    ref = (pre - pre.mean(-1, keepdims=True)) / np.sqrt(pre.var(-1, keepdims=True) + 1e-12) * g + be
+    Xd, Wd, bd, gd, bed, Rd = dev(X, torch.bfloat16), dev(Wt, torch.bfloat16), dev(b), dev(g), dev(be), dev(R)
+    ws = torch.zeros(pb.lib.cubert_gemm_layernorm_workspace_bytes(M) // 4, dtype=torch.int32, device="cuda")
+    fused = torch.full((M, N), float("nan"), device="cuda")
+    pb.check(pb.lib.cubert_op_gemm_residual_layernorm(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Rd.data_ptr(), gd.data_ptr(),
+                                                      bed.data_ptr(), fused.data_ptr(), None, ws.data_ptr(), M, N, K, K, tile, 0,
+                                                      stream()))
+    y = torch.full((M, N), float("nan"), device="cuda")
+    pb.check(pb.lib.cubert_op_gemm_residual(Xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), Rd.data_ptr(), y.data_ptr(), M, N, K, K,
+                                            BF16, tile if tile else 256, 0, stream()))
+    two = torch.full((M, N), float("nan"), device="cuda")
+    pb.check(pb.lib.cubert_op_add_layernorm(two.data_ptr(), y.data_ptr(), F32, gd.data_ptr(), bed.data_ptr(), None, M, N,
+                                            LN_NO_RESIDUAL, stream()))
+    torch.cuda.synchronize()
+    assert int(ws[0].item()) == 0
+    got = fused.cpu().numpy()
+    assert np.abs(got - ref).max() < 1e-3, np.abs(got - ref).max()
+    assert np.array_equal(got, two.cpu().numpy())

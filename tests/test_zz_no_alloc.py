@@ -62,3 +62,40 @@ def test_noalloc_refuses_what_does_not_fit(pb):
     rc = pb.lib.cubert_op_gemm_splitk_noalloc(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 64, 64, 64, 64,
                                               BF16, 17, 0, 0, st)
     assert rc != 0 and "splits" in pb.last_error()
+
+
+def test_noalloc_split_k_gemm_inside_a_captured_graph(pb):
+    """What the entry point is for: two calls recorded into one hipGraph (after an eager call that looks the scratch
+    address up), replayed several times with eager work in between; every replay gives the eager bits."""
+    rng = np.random.default_rng(7)
+    shapes = [(1600, 1024, 1024, 2), (200, 1024, 4096, 8)]
+    ops = []
+    for M, N, K, splits in shapes:
+        X = torch.from_numpy(rng.standard_normal((M, K), dtype=np.float32)).to(torch.bfloat16).cuda()
+        Wt = torch.from_numpy(rng.standard_normal((N, K), dtype=np.float32) * 0.05).to(torch.bfloat16).cuda()
+        bias = torch.from_numpy(rng.standard_normal(N, dtype=np.float32)).cuda()
+        ops.append((X, Wt, bias, torch.empty((M, N), device="cuda"), M, N, K, splits))
+
+    def enqueue(st):
+        for X, Wt, bias, Y, M, N, K, splits in ops:
+            pb.check(pb.lib.cubert_op_gemm_splitk_noalloc(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), M, N, K, K,
+                                                          BF16, splits, 0, 0, st))
+
+    enqueue(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    eager = [op[3].clone() for op in ops]
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        g.capture_begin()
+        enqueue(side.cuda_stream)
+        g.capture_end()
+    for rep in range(3):
+        for op in ops:
+            op[3].fill_(float("nan"))
+        run_pair(pb, BF16, 77, 128, 512, 2, 10 + rep)      # eager work on the shared scratch between replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for op, want in zip(ops, eager):
+            assert torch.equal(op[3], want), rep
