@@ -17,7 +17,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libcudaBERT.so")
-SOURCES = ["npy.cc", "weights.cc", "engine.cc", "capi.cc", "gemm.hip", "gemm_bf16_256.hip", "attention.hip", "rowwise.hip", "noalloc.hip"]
+SOURCES = ["npy.cc", "weights.cc", "engine.cc", "capi.cc", "gemm.hip", "gemm_bf16_256.hip", "gemm_bf16_128.hip", "attention.hip", "rowwise.hip", "noalloc.hip"]
 
 # -packed-fp32-ops is switched off: the compiler must not form packed FP32 math.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -524,14 +524,17 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
 
     // Short batches: the two GEMMs with only `hidden` output features have too few tiles for the
     // chip; they split K over several workgroups and the LayerNorm that follows adds the parts.
-    auto splits_for = [&](int K) {
-        const long tiles = (long)((N + 63) / 64) * ((H + 63) / 64);
-        int sp = 1;
-        if (cur_parts_ != 1 || !opt_.split_k) return sp;    // the parts of a split batch sit side by side in y32
-        while (sp < 16 && tiles * sp < 512 && K / (sp * 2) >= 256 && (long)(sp * 2) * N <= (long)N + kSplitRows) sp *= 2;
-        return sp;
+    // (Not for the parts of a split batch, which sit side by side in y32; the parts of K need rows of y32.)
+    auto plan_for = [&](int K) {
+        int max_splits = 1;
+        if (cur_parts_ == 1 && opt_.split_k) {
+            max_splits = 16;
+            while (max_splits > 1 && (long)max_splits * N > (long)N + kSplitRows) max_splits /= 2;
+        }
+        return gemm_plan(N, H, K, elt, max_splits, true, false);
     };
-    const int sp_ao = splits_for(H), sp_fo = splits_for(I);
+    const GemmPlan plan_ao = plan_for(H), plan_fo = plan_for(I);
+    const int sp_ao = plan_ao.splits, sp_fo = plan_fo.splits;
     // the attn-out / FFN-out GEMMs add the residual stream in their epilogue, so LayerNorm reads one operand
     const bool fuse_res = opt_.fuse_residual;
     // ... and, where the GEMM kernel can, normalise there as well: x32 and its bf16 copy come straight out of
@@ -566,7 +569,8 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;
         g.M = N; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_ao;
         g.residual = fuse_res ? x32 : nullptr;
-        if (ln_ao) { g.Y = x32; g.ln_gamma = L.g1; g.ln_beta = L.be1; g.ln_xb = xb; g.ln_xb_packed = pk; g.ln_ws = ln_ws; }
+        g.tile = plan_ao.tile;
+        if (ln_ao) { g.tile = 0; g.Y = x32; g.ln_gamma = L.g1; g.ln_beta = L.be1; g.ln_xb = xb; g.ln_xb_packed = pk; g.ln_ws = ln_ws; }
         if (!mark(kPhAttnOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
         if (!ln_ao && !launch_add_layernorm(x32, y32, kF32, L.g1, L.be1, xb, pk, N, H, st, sp_ao, !fuse_res)) return false;
@@ -579,7 +583,8 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
         g.elt = elt; g.out_elt = kF32; g.X = h; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = y32;
         g.M = N; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk; g.splits = sp_fo;
         g.residual = fuse_res ? x32 : nullptr;
-        if (ln_fo) { g.Y = x32; g.ln_gamma = L.g2; g.ln_beta = L.be2; g.ln_xb = xb; g.ln_xb_packed = pk; g.ln_ws = ln_ws; }
+        g.tile = plan_fo.tile;
+        if (ln_fo) { g.tile = 0; g.Y = x32; g.ln_gamma = L.g2; g.ln_beta = L.be2; g.ln_xb = xb; g.ln_xb_packed = pk; g.ln_ws = ln_ws; }
         if (!mark(kPhFFNOut) || !launch_gemm(g, st)) return false;
         if (!mark(kPhLayerNorm)) return false;
         if (!ln_fo && !launch_add_layernorm(x32, y32, kF32, L.g2, L.be2, xb, pk, N, H, st, sp_fo, !fuse_res)) return false;

@@ -38,6 +38,8 @@ namespace cubert {
 
 bool launch_gemm_bf16_t256(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
 bool launch_gemm_bf16_t256x128(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
+bool launch_gemm_bf16_t128(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
+bool launch_gemm_bf16_t256x128_deep(const gemm_detail::GemmDev& d, int out_elt, int epilogue, hipStream_t stream);
 int gemm_pick_tile(int M, int N, int K, int elt);
 int gemm_ln_pick_tile(int M, int N, int K, int elt);
 
@@ -360,6 +362,71 @@ int gemm_pick_tile(int M, int N, int K, int elt) {
     return bt;
 }
 
+// Tile and split count for a problem (tile as in GemmParams::tile, never 0).  max_splits > 1: the caller can take the
+// result as that many partial sums (float32 result, plain bias epilogue; see GemmParams::splits).
+//
+// Below kPlanSmallRows rows of bf16 operands the launch does not fill the chip for long and what counts is how the
+// workgroups spread over the 256 CUs.  Estimated time (microseconds, constants measured on MI355X with launches of
+// a few hundred to a few thousand rows of the four linears of BERT-large) = launch + result traffic + T * g, where T is the time of a
+// workgroup that has its CU to itself (a constant plus a cost per half-step of 32 k), and g says how the launch
+// stretches when a CU gets w > 1 workgroups on average: g = 1 + (w - 1 + q) * rho; rho is what one more workgroup on a CU
+// costs relative to a lone one (1: nothing is gained from sharing a CU, the 128 x 128 tile saturates the LDS on its
+// own) and q allows for the uneven hand-out of coarse tiles.  From kPlanSmallRows rows on, and for float32 operands,
+// gemm_pick_tile decides (its costs were measured inside whole forward passes at the power limit) and K is not split.
+constexpr int kPlanSmallRows = 6144;
+
+namespace {
+// Best (tile, splits) with min_splits <= splits <= max_splits (powers of two times min_splits).
+GemmPlan plan_small(int M, int N, int K, int min_splits, int max_splits, bool f32_result, bool gelu) {
+    // launch: before the first workgroup runs; fixed + per_hs * half-steps: a workgroup alone on its CU (deep_k: what a
+    // half-step costs more when K > 2048 and the weights stream from memory); rho, q: see above; out: weight of the
+    // result traffic (bytes / 4 TB/s).  Least-squares fit (5 % mean error) to launches of the four linears of BERT-large
+    // at 400 .. 6400 rows that cycle through 40 weight matrices, so that weights come from memory as in a forward pass.
+    struct Cand { int tile, bm, bn; double launch, fixed, per_hs, rho, q, out, deep_k; bool splits, k128; };
+    static const Cand cands[] = {
+        {64, 64, 64, 2.80, 0.20, 0.129, 0.77, 0.37, 0.01, 0.02, true, false},
+        {kTile128Hand, 128, 128, 2.37, 2.81, 0.283, 0.61, 0.16, 0.28, 0.14, true, false},
+        {kTile256x128, 128, 256, 8.00, 0.95, 0.260, 1.21, 0.45, 0.86, 0.46, false, false},
+        {kTile256x128Deep, 128, 256, 6.25, 1.33, 0.263, 1.50, 0.62, 0.86, 0.43, false, true},
+        {256, 256, 256, 8.00, 3.43, 0.448, 1.15, 0.85, 0.97, 0.11, false, true},
+    };
+    GemmPlan best{64, min_splits};
+    double best_cost = 1e30;
+    for (const Cand& c : cands) {
+        if ((!c.splits && min_splits > 1) || (c.k128 && K % 128 != 0)) continue;
+        for (int sp = min_splits; sp <= (c.splits ? max_splits : 1) && sp <= 16; sp *= 2) {
+            if (sp > min_splits && K / sp < 128) break;             // at least four half-steps per share
+            const double wgs = (double)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * sp;
+            const double w = wgs / 256.0;
+            const double g = w <= 1.0 ? 1.0 : 1.0 + (w - 1.0 + c.q) * c.rho;
+            const double T = c.fixed + c.per_hs * (K / 32.0 / sp) * (K > 2048 ? 1.0 + c.deep_k : 1.0) + (sp > 1 ? 0.6 : 0.0) +
+                             (gelu ? 0.8 : 0.0);
+            const double out_us = (double)M * N * (f32_result ? 4.0 : 2.0) * sp / 4.0e6;
+            // the consumer of split results reads every part again
+            const double cost = c.launch + c.out * out_us * (sp > 1 ? 1.5 : 1.0) + T * g;
+            if (cost < best_cost) { best_cost = cost; best = GemmPlan{c.tile, sp}; }
+        }
+    }
+    return best;
+}
+}  // namespace
+
+GemmPlan gemm_plan(int M, int N, int K, int elt, int max_splits, bool f32_result, bool gelu) {
+    GemmPlan best{gemm_pick_tile(M, N, K, elt), 1};
+    if (elt != kBF16 || M >= kPlanSmallRows || K % 64 != 0) {
+        if (max_splits > 1) {
+            // float32 operands: the rule the short batches were tuned with (64 x 64 tiles, at most 512 workgroups)
+            const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
+            int sp = 1;
+            while (sp * 2 <= max_splits && tiles * sp < 512 && K / (sp * 2) >= 256) sp *= 2;
+            best.splits = sp;
+            if (sp > 1 && best.tile == 256) best.tile = 128;      // the 256 x 256 kernel does not split
+        }
+        return best;
+    }
+    return plan_small(M, N, K, 1, max_splits > 1 ? max_splits : 1, f32_result, gelu);
+}
+
 bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     const int es = (p.elt == kBF16) ? 2 : 4;
     const int bk = 128 / es;
@@ -449,16 +516,34 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
             return false;
         }
     }
-    int bt = p.tile ? p.tile : gemm_pick_tile(p.M, p.N, p.K, p.elt);
+    int bt = p.tile;
+    if (!bt) {
+        // the caller has settled on the split count; the tile follows
+        if (p.elt == kBF16 && p.M < kPlanSmallRows && p.K % 64 == 0)
+            bt = plan_small(p.M, p.N, p.K, d.splits, d.splits, out == kF32, epi == kEpiBiasGelu).tile;
+        else
+            bt = gemm_pick_tile(p.M, p.N, p.K, p.elt);
+    }
     if (epi == kEpiBiasResLN && !p.tile) bt = gemm_ln_pick_tile(p.M, p.N, p.K, p.elt);
-    if (d.splits > 1 && bt == 256 && !p.tile) bt = 128;      // the hand-scheduled kernel does not split
+    if (d.splits > 1 && (bt == 256 || bt == kTile256x128 || bt == kTile256x128Deep) && !p.tile) bt = 128;      // those kernels do not split
     if (epi == kEpiBiasResLN && p.compiler_scheduled) { set_error("gemm: the LayerNorm epilogue has no compiler-scheduled kernel"); return false; }
-    if (bt == kTile256x128) {
+    if (bt == kTile256x128 || bt == kTile256x128Deep) {
         if (p.elt != kBF16 || d.splits != 1) { set_error("gemm: the 256x128 tile is bf16 only and does not split K"); return false; }
         d.tiles_n = (p.N + 255) / 256;
         d.tiles_m = (p.M + 127) / 128;
         d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 8);
+        if (bt == kTile256x128Deep) {
+            if (epi == kEpiBiasResLN) { set_error("gemm: the one-per-CU 256x128 tile has no LayerNorm epilogue"); return false; }
+            return launch_gemm_bf16_t256x128_deep(d, out, epi, stream);
+        }
         return launch_gemm_bf16_t256x128(d, out, epi, stream);
+    }
+    if (bt == kTile128Hand) {
+        if (p.elt != kBF16) { set_error("gemm: the hand-scheduled 128 tile is bf16 only"); return false; }
+        d.tiles_n = (p.N + 127) / 128;
+        d.tiles_m = (p.M + 127) / 128;
+        d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 8);
+        return launch_gemm_bf16_t128(d, out, epi, stream);
     }
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;

@@ -4,6 +4,8 @@ string) of the bf16 GEMM macro tiles:
 
     python gen_gemm_asm.py      > gemm_bf16_256_loop.inc        # 256 x 256, one workgroup per CU
     python gen_gemm_asm.py half > gemm_bf16_256x128_loop.inc    # 256 x 128, two per CU (end of file)
+    python gen_gemm_asm.py quarter > gemm_bf16_128_loop.inc     # 128 x 128, three per CU (end of file)
+    python gen_gemm_asm.py deep > gemm_bf16_256x128_deep_loop.inc  # 256 x 128, one per CU, the 256 x 256 pipeline
 
 The rest of this comment describes the 256 x 256 loop.
 
@@ -42,12 +44,6 @@ in slot c ^ ((r >> 2) & 3), which spreads the fragment reads of any
 16 rows (64 lanes x 16 B) to M0 + 16 * lane; the swizzle is applied on the
 global side (which chunk a lane fetches).
 """
-WA, XA, WB, XB = 112, 128, 144, 160
-ADDR = 96             # + 4 * bank + {0: W kk0, 1: W kk1, 2: X kk0, 3: X kk1}
-W_VOFF, X_VOFF = 104, 108
-NSTAGE = 4
-
-
 def vreg4(base):
     return "v[%d:%d]" % (base, base + 3)
 
@@ -83,68 +79,78 @@ class Emitter:
         self.guaranteed = None
 
 
-READ_ORDER = [("w", 0), ("x", 0), ("x", 1), ("x", 2), ("x", 3), ("w", 1), ("w", 2), ("w", 3)]
-
-
-def frag_reads(stage, kk, wset, xset):
-    bank, half = stage >> 1, stage & 1
-    out = []
-    for kind, b in READ_ORDER:
-        if kind == "w":
-            out.append((wset + 4 * b, ADDR + 4 * bank + kk, half * 32768 + b * 2048))
-        else:
-            out.append((xset + 4 * b, ADDR + 4 * bank + 2 + kk, half * 32768 + b * 2048))
-    return out
-
-
-def dma_instrs(stage):
-    """The eight global->LDS loads of one tile into `stage`: (M0 update, load)."""
-    out = []
-    for k in range(8):
-        m0 = ("s_mov_b32 m0, s%d" % (92 + stage)) if k == 0 else "s_add_u32 m0, m0, 0x1000"
-        if k < 4:
-            ld = "buffer_load_dwordx4 v%d, %%[wres], s96 offen lds" % (W_VOFF + k)
-        else:
-            ld = "buffer_load_dwordx4 v%d, %%[xres], s98 offen lds" % (X_VOFF + k - 4)
-        out.append((m0, ld))
-    return out
-
-
+NSTAGE = 4
 DMA_EVERY = 2         # one global->LDS load behind every second MFMA
 
 
-def half_step(e, stage, dma, prefetch_next, vmcnt, barrier):
-    """One half-step on `stage`.  On entry the 8 reads of set A (k-phase 0 of this
-    tile) have been issued, in READ_ORDER, as the latest 8 LDS reads."""
-    e.emit("; ---- half-step on stage %d%s" % (stage, ", fetch into stage %d" % ((stage + 3) % NSTAGE) if dma else ""))
-    dmas = dma_instrs((stage + 3) % NSTAGE) if dma else []
-    for kk in range(2):
-        wset, xset = (WA, XA) if kk == 0 else (WB, XB)
-        if kk == 0:
-            pending = frag_reads(stage, 1, WB, XB)
-        else:
-            pending = frag_reads((stage + 1) % NSTAGE, 0, WA, XA) if prefetch_next else []
-        m = 0
-        for i in range(4):
-            for j in range(4):
-                e.need(wset + 4 * i, xset + 4 * j)
-                gm = 16 * kk + m
-                d = gm // DMA_EVERY if (dmas and gm % DMA_EVERY == 0 and gm // DMA_EVERY < 8) else None
-                if d is not None:
-                    e.emit(dmas[d][0])      # M0 update in front of the MFMA: the MFMA is the
-                e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %   # wait state before M0 is used
-                       (i, j, vreg4(wset + 4 * i), vreg4(xset + 4 * j), i, j))
-                if d is not None:
-                    e.emit(dmas[d][1])
-                # The destination set of these reads was last used by MFMAs of the
-                # previous k-phase, all of which have issued.
-                if m < len(pending):
-                    e.read(*pending[m])
-                m += 1
-    if vmcnt is not None:
-        e.emit("s_waitcnt vmcnt(%d)" % vmcnt)
-    if barrier:
-        e.emit("s_barrier")
+class Deep:
+    """Register and LDS plan of the four-stage loop described above, for a wave tile of nwb x nxb accumulator
+    blocks (32 features x 32 tokens each).  The 256 x 256 kernel is 4 x 4; "deep" mode builds the 256 x 128 tile
+    (4 x 2, end of file) the same way."""
+
+    def __init__(self, name, nwb, nxb, wa, xa, wb, xb, addr, wvoff, xvoff, stage):
+        self.name, self.nwb, self.nxb = name, nwb, nxb
+        self.wa, self.xa, self.wb, self.xb = wa, xa, wb, xb
+        self.addr, self.wvoff, self.xvoff, self.stage = addr, wvoff, xvoff, stage
+        self.ndma = nwb + nxb            # global->LDS loads per tile and wave = fragment reads per k-phase
+        # the pair the first MFMA needs first, then the other X fragments, then the other W fragments
+        self.read_order = [("w", 0)] + [("x", b) for b in range(nxb)] + [("w", b) for b in range(1, nwb)]
+
+    def frag_reads(self, stage, kk, wset, xset):
+        bank, half = stage >> 1, stage & 1
+        out = []
+        for kind, b in self.read_order:
+            if kind == "w":
+                out.append((wset + 4 * b, self.addr + 4 * bank + kk, half * self.stage + b * 2048))
+            else:
+                out.append((xset + 4 * b, self.addr + 4 * bank + 2 + kk, half * self.stage + b * 2048))
+        return out
+
+    def dma_instrs(self, stage):
+        """The global->LDS loads of one tile into `stage`: (M0 update, load)."""
+        out = []
+        for k in range(self.ndma):
+            m0 = ("s_mov_b32 m0, s%d" % (92 + stage)) if k == 0 else "s_add_u32 m0, m0, 0x1000"
+            if k < self.nwb:
+                ld = "buffer_load_dwordx4 v%d, %%[wres], s96 offen lds" % (self.wvoff + k)
+            else:
+                ld = "buffer_load_dwordx4 v%d, %%[xres], s98 offen lds" % (self.xvoff + k - self.nwb)
+            out.append((m0, ld))
+        return out
+
+    def half_step(self, e, stage, dma, prefetch_next, vmcnt, barrier):
+        """One half-step on `stage`.  On entry the reads of set A (k-phase 0 of this
+        tile) have been issued, in read_order, as the latest LDS reads."""
+        e.emit("; ---- half-step on stage %d%s" % (stage, ", fetch into stage %d" % ((stage + 3) % NSTAGE) if dma else ""))
+        dmas = self.dma_instrs((stage + 3) % NSTAGE) if dma else []
+        per_phase = self.nwb * self.nxb
+        for kk in range(2):
+            wset, xset = (self.wa, self.xa) if kk == 0 else (self.wb, self.xb)
+            if kk == 0:
+                pending = self.frag_reads(stage, 1, self.wb, self.xb)
+            else:
+                pending = self.frag_reads((stage + 1) % NSTAGE, 0, self.wa, self.xa) if prefetch_next else []
+            m = 0
+            for i in range(self.nwb):
+                for j in range(self.nxb):
+                    e.need(wset + 4 * i, xset + 4 * j)
+                    gm = per_phase * kk + m
+                    d = gm // DMA_EVERY if (dmas and gm % DMA_EVERY == 0 and gm // DMA_EVERY < self.ndma) else None
+                    if d is not None:
+                        e.emit(dmas[d][0])      # M0 update in front of the MFMA: the MFMA is the
+                    e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %   # wait state before M0 is used
+                           (i, j, vreg4(wset + 4 * i), vreg4(xset + 4 * j), i, j))
+                    if d is not None:
+                        e.emit(dmas[d][1])
+                    # The destination set of these reads was last used by MFMAs of the
+                    # previous k-phase, all of which have issued.
+                    if m < len(pending):
+                        e.read(*pending[m])
+                    m += 1
+        if vmcnt is not None:
+            e.emit("s_waitcnt vmcnt(%d)" % vmcnt)
+        if barrier:
+            e.emit("s_barrier")
 
 
 def advance_k(e):
@@ -153,44 +159,58 @@ def advance_k(e):
     e.emit("s_add_u32 s98, s98, %[xkstep]")
 
 
-def main():
+FULL = Deep("", 4, 4, 112, 128, 144, 160, 96, 104, 108, 0x8000)
+# "deep" mode: python gen_gemm_asm.py deep > gemm_bf16_256x128_deep_loop.inc
+# The 256 x 128 tile (4 x 2 accumulator blocks per wave) with the pipeline of the 256 x 256 loop: four stages of
+# 24 KiB (W tile at +0, X tile at +0x4000, which the kernel puts into %[xb]), loads three half-steps ahead, no
+# fragment read waited for right after issue.  96 KiB of LDS: one workgroup per CU, which is what a launch of at
+# most 256 workgroups gets anyway; there the two-per-CU loop ("half" mode) leaves the matrix pipe idle half of the
+# time, because nothing runs beside it while it waits for the last fragment reads of a half-step and the barrier.
+#   v64..v79 / v80..v87  W / X fragments, set A      v88..v103 / v104..v111  set B
+#   v112..v119  fragment row addresses (stages 0-1, 2-3)   v120..v123 / v124..v125  W / X lane offsets
+DEEP = Deep("deep", 4, 2, 64, 80, 88, 104, 112, 120, 124, 0x6000)
+
+
+def main(c=FULL):
     e = Emitter()
     e.emit("; ======== setup ========")
-    e.emit("v_mov_b32 v%d, %%[wb]" % (ADDR + 0))
-    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (ADDR + 1))
-    e.emit("v_mov_b32 v%d, %%[xb]" % (ADDR + 2))
-    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (ADDR + 3))
+    e.emit("v_mov_b32 v%d, %%[wb]" % (c.addr + 0))
+    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (c.addr + 1))
+    e.emit("v_mov_b32 v%d, %%[xb]" % (c.addr + 2))
+    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (c.addr + 3))
     for r in range(4):
-        e.emit("v_add_u32 v%d, 0x10000, v%d" % (ADDR + 4 + r, ADDR + r))
-    e.emit("v_mov_b32 v%d, %%[wv0]" % W_VOFF)
-    e.emit("v_mov_b32 v%d, %%[xv0]" % X_VOFF)
-    for i in range(1, 4):
-        e.emit("v_add_u32 v%d, %%[w64], v%d" % (W_VOFF + i, W_VOFF + i - 1))
-        e.emit("v_add_u32 v%d, %%[x64], v%d" % (X_VOFF + i, X_VOFF + i - 1))
+        e.emit("v_add_u32 v%d, 0x%x, v%d" % (c.addr + 4 + r, 2 * c.stage, c.addr + r))
+    e.emit("v_mov_b32 v%d, %%[wv0]" % c.wvoff)
+    e.emit("v_mov_b32 v%d, %%[xv0]" % c.xvoff)
+    for i in range(1, max(c.nwb, c.nxb)):
+        if i < c.nwb:
+            e.emit("v_add_u32 v%d, %%[w64], v%d" % (c.wvoff + i, c.wvoff + i - 1))
+        if i < c.nxb:
+            e.emit("v_add_u32 v%d, %%[x64], v%d" % (c.xvoff + i, c.xvoff + i - 1))
     # zero the accumulators: 0 * 0 + 0 through the matrix pipe (the accumulator
     # operands are write-only for the compiler, which halves the operand count)
     for r in range(4):
-        e.emit("v_mov_b32 v%d, 0" % (WA + r))
+        e.emit("v_mov_b32 v%d, 0" % (c.wa + r))
     e.emit("s_nop 7")      # VALU result -> MFMA source operand needs wait states the assembler does not add
-    for i in range(4):
-        for j in range(4):
-            e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, 0" % (i, j, vreg4(WA), vreg4(WA)))
+    for i in range(c.nwb):
+        for j in range(c.nxb):
+            e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, 0" % (i, j, vreg4(c.wa), vreg4(c.wa)))
     e.emit("s_mov_b32 s92, %[m0b]")
     for s in range(1, NSTAGE):
-        e.emit("s_add_u32 s%d, s%d, 0x8000" % (92 + s, 92 + s - 1))
+        e.emit("s_add_u32 s%d, s%d, 0x%x" % (92 + s, 92 + s - 1, c.stage))
     e.emit("; ======== prologue: tiles 0, 1, 2 -> stages 0, 1, 2 ========")
     e.emit("s_mov_b32 s96, 0")
     e.emit("s_mov_b32 s98, 0")
     for t in range(3):
-        for m0, ld in dma_instrs(t):
+        for m0, ld in c.dma_instrs(t):
             e.emit(m0)
             e.emit("s_nop 0")
             e.emit(ld)
         if t < 2:
             advance_k(e)
-    e.emit("s_waitcnt vmcnt(8)")          # tiles 0 and 1 have landed
+    e.emit("s_waitcnt vmcnt(%d)" % c.ndma)          # tiles 0 and 1 have landed
     e.emit("s_barrier")
-    for r in frag_reads(0, 0, WA, XA):
+    for r in c.frag_reads(0, 0, c.wa, c.xa):
         e.read(*r)
     e.emit("s_mov_b32 s97, 4")
     e.emit("s_cmp_ge_u32 s97, %[ht]")
@@ -198,7 +218,7 @@ def main():
     e.emit("L_loop_%=:")
     for s in range(NSTAGE):
         advance_k(e)
-        half_step(e, s, dma=True, prefetch_next=True, vmcnt=8, barrier=True)
+        c.half_step(e, s, dma=True, prefetch_next=True, vmcnt=c.ndma, barrier=True)
     e.forget_bound()                       # the loop head is reached from two places
     e.emit("s_add_u32 s97, s97, 4")
     e.emit("s_cmp_lt_u32 s97, %[ht]")
@@ -206,11 +226,11 @@ def main():
     e.emit("L_tail_%=:")
     e.forget_bound()
     advance_k(e)
-    half_step(e, 0, dma=True, prefetch_next=True, vmcnt=8, barrier=True)      # fetches the last tile
-    half_step(e, 1, dma=False, prefetch_next=True, vmcnt=0, barrier=True)
-    half_step(e, 2, dma=False, prefetch_next=True, vmcnt=None, barrier=False)
-    half_step(e, 3, dma=False, prefetch_next=False, vmcnt=None, barrier=False)
-    print("// Generated by gen_gemm_asm.py -- do not edit.")
+    c.half_step(e, 0, dma=True, prefetch_next=True, vmcnt=c.ndma, barrier=True)      # fetches the last tile
+    c.half_step(e, 1, dma=False, prefetch_next=True, vmcnt=0, barrier=True)
+    c.half_step(e, 2, dma=False, prefetch_next=True, vmcnt=None, barrier=False)
+    c.half_step(e, 3, dma=False, prefetch_next=False, vmcnt=None, barrier=False)
+    print("// Generated by gen_gemm_asm.py%s -- do not edit." % (" " + c.name if c.name else ""))
     for ln in e.lines:
         print('"%s\\n"' % ln)
 
@@ -240,51 +260,74 @@ def main():
 # vmcnt(6) (everything but the loads just issued, i.e. tile h+1, has landed); barrier.  Loads
 # issued for tiles past the end of K fetch the last tile again and are never used; the
 # block ends with vmcnt(0) and a barrier so that nothing lands in the LDS afterwards.
-H_WA, H_XA, H_WB, H_XB = 64, 80, 88, 104
-H_BASE, H_CUR = 112, 122
-H_WVOFF, H_XVOFF = 116, 120
-H_STAGE = 0x6000
+class Skewed:
+    """Register and LDS plan of a loop whose body is one skewed half-step (see above): `nw` accumulator block
+    rows (32 features each) per wave; two block columns (64 tokens)."""
+
+    def __init__(self, name, nw, wa, xa, wb, xb, base, cur, wvoff, xvoff, x_lds, stage, nstage=3):
+        self.name, self.nw, self.nstage = name, nw, nstage
+        self.wa, self.xa, self.wb, self.xb = wa, xa, wb, xb
+        self.base, self.cur, self.wvoff, self.xvoff = base, cur, wvoff, xvoff
+        self.x_lds, self.stage = x_lds, stage
+        self.n = nw + 2            # fragment reads per k-phase = global->LDS loads per tile and wave
 
 
-def main_half():
+HALF = Skewed("half", 4, 64, 80, 88, 104, 112, 122, 116, 120, 0x4000, 0x6000)
+# 128 x 128 macro tile, three workgroups per CU ("quarter" mode):
+#     python gen_gemm_asm.py quarter > gemm_bf16_128_loop.inc
+# The same loop with a W tile of 128 rows: a wave owns 64 features x 64 tokens = 2 x 2 accumulator blocks
+# (64 AGPRs) and everything the block writes lies below v92, so a SIMD holds three waves of three
+# workgroups; three LDS stages of 16 KiB (W tile at +0, X tile at +0x2000).  Per half-step a wave issues
+# 8 MFMAs, 8 fragment reads and 4 global->LDS loads.  For problems too small to fill the chip with the
+# larger tiles.  The K offsets start at %[wk0] / %[xk0] (split K: a workgroup's share of K).
+#   v48..v55 / v56..v63  W / X fragments, set A      v64..v71 / v72..v79  set B
+#   v80..v83  fragment row addresses in stage 0      v84..v87  the same for the current stage
+#   v88..v89 / v90..v91  W / X lane offsets
+QUARTER = Skewed("quarter", 2, 48, 56, 64, 72, 80, 84, 88, 90, 0x2000, 0x4000)
+
+
+def main_skewed(c):
+    quarter = c.name == "quarter"
     e = Emitter()
     e.emit("; ======== setup ========")
-    e.emit("v_mov_b32 v%d, %%[wb]" % (H_BASE + 0))
-    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (H_BASE + 1))
-    e.emit("v_mov_b32 v%d, %%[xb]" % (H_BASE + 2))
-    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (H_BASE + 3))
-    e.emit("v_mov_b32 v%d, %%[wv0]" % H_WVOFF)
-    e.emit("v_mov_b32 v%d, %%[xv0]" % H_XVOFF)
-    for i in range(1, 4):
-        e.emit("v_add_u32 v%d, %%[w64], v%d" % (H_WVOFF + i, H_WVOFF + i - 1))
-    e.emit("v_add_u32 v%d, %%[x64], v%d" % (H_XVOFF + 1, H_XVOFF))
+    e.emit("v_mov_b32 v%d, %%[wb]" % (c.base + 0))
+    e.emit("v_xor_b32 v%d, 0x20, %%[wb]" % (c.base + 1))
+    e.emit("v_mov_b32 v%d, %%[xb]" % (c.base + 2))
+    e.emit("v_xor_b32 v%d, 0x20, %%[xb]" % (c.base + 3))
+    e.emit("v_mov_b32 v%d, %%[wv0]" % c.wvoff)
+    e.emit("v_mov_b32 v%d, %%[xv0]" % c.xvoff)
+    for i in range(1, c.nw):
+        e.emit("v_add_u32 v%d, %%[w64], v%d" % (c.wvoff + i, c.wvoff + i - 1))
+    e.emit("v_add_u32 v%d, %%[x64], v%d" % (c.xvoff + 1, c.xvoff))
     for r in range(4):
-        e.emit("v_mov_b32 v%d, 0" % (H_WA + r))
+        e.emit("v_mov_b32 v%d, 0" % (c.wa + r))
     e.emit("s_nop 7")      # VALU result -> MFMA source operand
-    for i in range(4):
+    for i in range(c.nw):
         for j in range(2):
-            e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, 0" % (i, j, vreg4(H_WA), vreg4(H_WA)))
+            e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, 0" % (i, j, vreg4(c.wa), vreg4(c.wa)))
     e.emit("s_mov_b32 s94, %[m0b]")
     e.emit("s_mov_b32 s92, 0")
     e.emit("s_mov_b32 s93, 0")
-    e.emit("s_mov_b32 s96, 0")
-    e.emit("s_mov_b32 s98, 0")
+    e.emit("s_mov_b32 s96, %s" % ("%[wk0]" if quarter else "0"))
+    e.emit("s_mov_b32 s98, %s" % ("%[xk0]" if quarter else "0"))
 
     def dma(k):
-        """k-th of the wave's six loads of the tile at stage offset s93: (M0 update, load)."""
+        """k-th of the wave's loads of the tile at stage offset s93: (M0 update, load)."""
         m0 = "s_add_u32 m0, s94, s93" if k == 0 else "s_add_u32 m0, m0, 0x1000"
-        if k < 4:
-            ld = "buffer_load_dwordx4 v%d, %%[wres], s96 offen lds" % (H_WVOFF + k)
+        if k < c.nw:
+            ld = "buffer_load_dwordx4 v%d, %%[wres], s96 offen lds" % (c.wvoff + k)
         else:
-            ld = "buffer_load_dwordx4 v%d, %%[xres], s98 offen lds" % (H_XVOFF + k - 4)
+            ld = "buffer_load_dwordx4 v%d, %%[xres], s98 offen lds" % (c.xvoff + k - c.nw)
         return m0, ld
 
     def rotate(reg):
-        e.emit("s_add_u32 s%d, s%d, 0x%x" % (reg, reg, H_STAGE))
-        e.emit("s_cmp_eq_u32 s%d, 0x%x" % (reg, 3 * H_STAGE))
+        e.emit("s_add_u32 s%d, s%d, 0x%x" % (reg, reg, c.stage))
+        e.emit("s_cmp_eq_u32 s%d, 0x%x" % (reg, c.nstage * c.stage))
         e.emit("s_cselect_b32 s%d, 0, s%d" % (reg, reg))
 
-    e.emit("; ======== prologue: tiles 0, 1 -> stages 0, 1 ========")
+    e.emit("; ======== prologue: tiles 0, 1 -> stages 0, 1 ========" if c.nstage == 3 else
+           "; ======== prologue: tiles 0 .. %d -> stages 0 .. %d ========" % (c.nstage - 2, c.nstage - 2))
+    ahead = c.n * (c.nstage - 2)      # loads of the tiles that need not have landed when a half-step ends
     def advance_k_clamped():
         # The loads run two tiles ahead of the multiply, so the last two half-steps ask for tiles
         # past the end of K: they fetch the last tile again (the range check of a buffer
@@ -293,37 +336,37 @@ def main_half():
         e.emit("s_min_u32 s96, s96, %[wkmax]")
         e.emit("s_min_u32 s98, s98, %[xkmax]")
 
-    for t in range(2):
-        for k in range(6):
+    for t in range(c.nstage - 1):
+        for k in range(c.n):
             m0, ld = dma(k)
             e.emit(m0)
             e.emit("s_nop 0")
             e.emit(ld)
         rotate(93)
         advance_k_clamped()
-    e.emit("s_waitcnt vmcnt(6)")           # tile 0 has landed
+    e.emit("s_waitcnt vmcnt(%d)" % ahead)         # tile 0 has landed
     e.emit("s_barrier")
 
     def reads(kk, wset, xset):
-        out = [(wset + 4 * b, H_CUR + kk, b * 2048) for b in range(4)]
-        out += [(xset + 4 * b, H_CUR + 2 + kk, 0x4000 + b * 2048) for b in range(2)]
+        out = [(wset + 4 * b, c.cur + kk, b * 2048) for b in range(c.nw)]
+        out += [(xset + 4 * b, c.cur + 2 + kk, c.x_lds + b * 2048) for b in range(2)]
         # first the pair the first MFMA needs
-        return [out[0], out[4], out[5], out[1], out[2], out[3]]
+        return [out[0], out[c.nw], out[c.nw + 1]] + out[1:c.nw]
 
     def cur_addresses():
         for r in range(4):
-            e.emit("v_add_u32 v%d, s92, v%d" % (H_CUR + r, H_BASE + r))
+            e.emit("v_add_u32 v%d, s92, v%d" % (c.cur + r, c.base + r))
 
     def mfmas(wset, xset, tracked, pending, dma_from):
-        """Eight MFMAs on one fragment set; `pending` LDS reads and the DMA loads
-        dma_from, dma_from + 1, dma_from + 2 go behind them."""
+        """The MFMAs on one fragment set; `pending` LDS reads and half of the tile's DMA loads, from
+        number dma_from on, go behind them."""
         n_dma = 0
         m = 0
-        for i in range(4):
+        for i in range(c.nw):
             for j in range(2):
                 if tracked:
                     e.need(wset + 4 * i, xset + 4 * j)
-                d = dma_from + n_dma if (dma_from is not None and m % 2 == 0 and n_dma < 3) else None
+                d = dma_from + n_dma if (dma_from is not None and m % 2 == 0 and n_dma < c.n // 2) else None
                 if d is not None:
                     e.emit(dma(d)[0])
                 e.emit("v_mfma_f32_32x32x16_bf16 %%[c%d%d], %s, %s, %%[c%d%d]" %
@@ -339,9 +382,9 @@ def main_half():
         rotate(92)
         rotate(93)
         advance_k_clamped()
-        # vmcnt(6): everything but the loads just issued, i.e. the next tile, has landed.
+        # vmcnt(n): everything but the loads just issued, i.e. the next tile, has landed.
         # lgkmcnt(0): my reads of this tile are done before anybody may overwrite its stage.
-        e.emit("s_waitcnt vmcnt(6) lgkmcnt(0)")
+        e.emit("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ahead)
         e.emit("s_barrier")
 
     # The pipeline is skewed by one k-phase: a half-step starts by reading its tile's k-phase-0
@@ -349,11 +392,11 @@ def main_half():
     # ago) while they arrive; then k-phase 0 on set A while k-phase 1 is read into set B.
     e.emit("; ======== half-step 0: no previous tile ========")
     cur_addresses()
-    for r in reads(0, H_WA, H_XA):
+    for r in reads(0, c.wa, c.xa):
         e.read(*r)
-    mfmas(H_WA, H_XA, True, reads(1, H_WB, H_XB), 0)
-    # the three remaining loads of tile 2 without MFMAs to hide behind
-    for k in range(3, 6):
+    mfmas(c.wa, c.xa, True, reads(1, c.wb, c.xb), 0)
+    # the remaining loads of tile 2 without MFMAs to hide behind
+    for k in range(c.n // 2, c.n):
         e.emit(dma(k)[0])
         e.emit("s_nop 0")
         e.emit(dma(k)[1])
@@ -363,13 +406,13 @@ def main_half():
     e.emit("s_cbranch_scc1 L_last_%=")
     e.emit("L_loop_%=:")
     cur_addresses()
-    for r in reads(0, H_WA, H_XA):
+    for r in reads(0, c.wa, c.xa):
         e.read(*r)
-    e.emit("s_waitcnt lgkmcnt(6)")         # set B (read during the previous half-step) is complete
+    e.emit("s_waitcnt lgkmcnt(%d)" % c.n)         # set B (read during the previous half-step) is complete
     e.forget_bound()
-    e.guaranteed = 6
-    mfmas(H_WB, H_XB, False, [], 0)
-    mfmas(H_WA, H_XA, True, reads(1, H_WB, H_XB), 3)
+    e.guaranteed = c.n
+    mfmas(c.wb, c.xb, False, [], 0)
+    mfmas(c.wa, c.xa, True, reads(1, c.wb, c.xb), c.n // 2)
     end_of_half_step()
     e.emit("s_add_u32 s97, s97, 1")
     e.emit("s_cmp_lt_u32 s97, %[ht]")
@@ -377,10 +420,10 @@ def main_half():
     e.emit("L_last_%=:")
     e.emit("s_waitcnt lgkmcnt(0)")
     e.emit("; ======== k-phase 1 of the last tile ========")
-    mfmas(H_WB, H_XB, False, [], None)
+    mfmas(c.wb, c.xb, False, [], None)
     e.emit("s_waitcnt vmcnt(0)")
     e.emit("s_barrier")
-    print("// Generated by gen_gemm_asm.py half -- do not edit.")
+    print("// Generated by gen_gemm_asm.py %s -- do not edit." % c.name)
     for ln in e.lines:
         print('"%s\\n"' % ln)
 
@@ -388,6 +431,14 @@ def main_half():
 if __name__ == "__main__":
     import sys
     if len(sys.argv) > 1 and sys.argv[1] == "half":
-        main_half()
+        if len(sys.argv) > 2:
+            HALF.nstage = int(sys.argv[2])
+        main_skewed(HALF)
+    elif len(sys.argv) > 1 and sys.argv[1] == "deep":
+        main(DEEP)
+    elif len(sys.argv) > 1 and sys.argv[1] == "quarter":
+        if len(sys.argv) > 2:
+            QUARTER.nstage = int(sys.argv[2])
+        main_skewed(QUARTER)
     else:
         main()

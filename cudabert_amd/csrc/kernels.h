@@ -37,6 +37,8 @@ struct Compact {
 };
 
 constexpr int kTile256x128 = 384;     // GemmParams::tile value of the 256 features x 128 tokens kernel
+constexpr int kTile256x128Deep = 385; // ... of the 256 x 128 kernel with one workgroup per CU and the deeper pipeline (K % 128 == 0)
+constexpr int kTile128Hand = 192;     // ... of the hand-scheduled 128 x 128 kernel (bf16, three workgroups per CU, splits K)
 
 struct GemmParams {
     const void* X = nullptr;
@@ -73,7 +75,7 @@ struct GemmParams {
     void* ln_xb = nullptr;
     bool ln_xb_packed = false;
     void* ln_ws = nullptr;
-    int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile) or kTile256x128
+    int tile = 0;             // 0 = choose; otherwise 64, 128 or 256 (square macro tile), kTile256x128 or kTile128Hand
     // Split K (kEpiBias, float32 Y): `splits` workgroups share a tile, each reduces its share of K and
     // writes its partial result to Y + z * M * N; the bias goes into partial 0.  The consumer adds
     // them up (launch_add_layernorm's y_parts).  Y must hold splits * M * N floats.
@@ -83,6 +85,11 @@ struct GemmParams {
     bool x_packed = false, w_packed = false, y_packed = false;
 };
 bool launch_gemm(const GemmParams& p, hipStream_t stream);
+// The tile (a GemmParams::tile value, never 0) and split count launch_gemm's cost model prefers for a problem.
+// max_splits > 1: the caller can take a float32 result as up to that many partial sums (a power of two is chosen).
+// f32_result / gelu: the launch will write float32 / use the GELU epilogue.
+struct GemmPlan { int tile; int splits; };
+GemmPlan gemm_plan(int M, int N, int K, int elt, int max_splits, bool f32_result, bool gelu);
 // Workspace of a GEMM with the LayerNorm in its epilogue (GemmParams::ln_ws) for up to M rows.
 size_t gemm_ln_workspace_bytes(size_t M);
 // Test aid: puts a workspace into a state in which the workgroups of row band 0 can never see their band complete

@@ -8,7 +8,8 @@ import pytest
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cudabert_amd", "csrc")
 
 
-@pytest.mark.parametrize("args,inc", [([], "gemm_bf16_256_loop.inc"), (["half"], "gemm_bf16_256x128_loop.inc")])
+@pytest.mark.parametrize("args,inc", [([], "gemm_bf16_256_loop.inc"), (["half"], "gemm_bf16_256x128_loop.inc"),
+                                      (["deep"], "gemm_bf16_256x128_deep_loop.inc"), (["quarter"], "gemm_bf16_128_loop.inc")])
 def test_inc_matches_generator(args, inc):
     out = subprocess.run([sys.executable, os.path.join(CSRC, "gen_gemm_asm.py")] + args, capture_output=True,
                          text=True, check=True).stdout
@@ -51,9 +52,10 @@ def _clobbers(hip_text, inc):
     return regs
 
 
-@pytest.mark.parametrize("inc", ["gemm_bf16_256_loop.inc", "gemm_bf16_256x128_loop.inc"])
-def test_every_register_the_loop_writes_is_declared_clobbered(inc):
+@pytest.mark.parametrize("inc,hip", [("gemm_bf16_256_loop.inc", "gemm_bf16_256.hip"), ("gemm_bf16_256x128_loop.inc", "gemm_bf16_256.hip"),
+                                     ("gemm_bf16_256x128_deep_loop.inc", "gemm_bf16_256.hip"), ("gemm_bf16_128_loop.inc", "gemm_bf16_128.hip")])
+def test_every_register_the_loop_writes_is_declared_clobbered(inc, hip):
     written = _written_registers(open(os.path.join(CSRC, inc)).read())
-    clob = _clobbers(open(os.path.join(CSRC, "gemm_bf16_256.hip")).read(), inc)
+    clob = _clobbers(open(os.path.join(CSRC, hip)).read(), inc)
     assert "m0" in written and "scc" in clob and "memory" in clob
     assert written <= clob, sorted(written - clob)

@@ -77,12 +77,14 @@ def gelu64(x):
 
 
 @pytest.mark.parametrize("elt", [F32, BF16])
-@pytest.mark.parametrize("tile", [64, 128, 256, 384])          # 384: the 256 x 128 two-per-CU kernel (bf16)
+@pytest.mark.parametrize("tile", [64, 128, 256, 384, 192, 385])     # 384 / 385: the 256 x 128 kernels (two / one per CU), 192: the hand-scheduled 128 tile (bf16)
 @pytest.mark.parametrize("M,N,K,epi", [(200, 128, 128, 0), (333, 384, 256, 1), (512, 1024, 1024, 0),
                                        (77, 512, 512, 2), (1000, 768, 3072, 0), (130, 256, 64, 0)])
 def test_gemm(pb, elt, tile, M, N, K, epi):
+    if tile == 385 and K % 128:
+        pytest.skip("the one-per-CU 256 x 128 kernel needs K to be a multiple of 128")
     print("gemm", elt, tile, M, N, K, epi, flush=True)
-    if tile == 384 and elt == F32:
+    if tile in (384, 192, 385) and elt == F32:
         pytest.skip("the 256 x 128 kernel is bf16 only")
     rng = np.random.default_rng(M * 7 + N + K + epi)
     X = rng.standard_normal((M, K)).astype(np.float32)
@@ -139,11 +141,11 @@ def test_gemm_rejects_bad_shapes(pb):
 
 @pytest.mark.parametrize("elt", [F32, BF16])
 @pytest.mark.parametrize("B,S,heads,tile", [(3, 33, 2, 64), (2, 200, 4, 128), (5, 128, 12, 256), (2, 200, 4, 384),
-                                            (5, 128, 12, 384)])
+                                            (5, 128, 12, 384), (2, 200, 4, 192), (5, 128, 12, 192), (2, 200, 4, 385), (5, 128, 12, 385)])
 @pytest.mark.parametrize("v_rowmajor", [0, 1])
 def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile, v_rowmajor):
     print("qkv", elt, B, S, heads, tile, v_rowmajor, flush=True)
-    if tile == 384 and elt == F32:
+    if tile in (384, 192, 385) and elt == F32:
         pytest.skip("the 256 x 128 kernel is bf16 only")
     rng = np.random.default_rng(B + S)
     H = heads * 64
@@ -372,10 +374,12 @@ def test_mask_softmax(pb, elt, B, R, S):
     assert (got[np.broadcast_to(mask[:, None, :] == 0, got.shape)] == 0).all()
 
 
-@pytest.mark.parametrize("tile,flags_extra", [(64, 0), (128, 0), (256, 0), (256, 8), (384, 0)])
+@pytest.mark.parametrize("tile,flags_extra", [(64, 0), (128, 0), (256, 0), (256, 8), (384, 0), (192, 0), (385, 0)])
 @pytest.mark.parametrize("M,N,K,epi,xp,wp,yp", [(200, 128, 128, 0, 1, 1, 0), (333, 384, 256, 1, 1, 1, 1), (512, 1024, 1024, 0, 1, 0, 0),
                                                (700, 512, 512, 0, 0, 1, 1), (1000, 768, 3072, 0, 1, 1, 0)])
 def test_gemm_packed_operands(pb, tile, flags_extra, M, N, K, epi, xp, wp, yp):
+    if tile == 385 and K % 128:
+        pytest.skip("the one-per-CU 256 x 128 kernel needs K to be a multiple of 128")
     """bf16 GEMM reading packed X / W and writing a packed Y; every kernel variant."""
     print("gemm packed", tile, flags_extra, M, N, K, epi, xp, wp, yp, flush=True)
     rng = np.random.default_rng(M + N + K)
@@ -409,10 +413,13 @@ def test_gemm_packed_operands(pb, tile, flags_extra, M, N, K, epi, xp, wp, yp):
 
 @pytest.mark.parametrize("elt", [F32, BF16])
 @pytest.mark.parametrize("M,N,K,splits,tile", [(200, 1024, 4096, 4, 64), (77, 128, 512, 2, 0), (300, 256, 1024, 8, 128),
-                                               (64, 64, 384, 3, 64)])
+                                               (64, 64, 384, 3, 64), (200, 1024, 4096, 8, 192), (1600, 1024, 1024, 4, 192),
+                                               (333, 384, 320, 5, 192)])
 def test_gemm_split_k_and_layernorm_of_parts(pb, elt, M, N, K, splits, tile):
     """Split-K GEMM: the partial results add up to the plain product, and the residual+LayerNorm
     kernel consumes them as its addend."""
+    if tile == 192 and elt == F32:
+        pytest.skip("the hand-scheduled 128 tile is bf16 only")
     rng = np.random.default_rng(M + K)
     X = rng.standard_normal((M, K)).astype(np.float32)
     Wt = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
@@ -513,7 +520,7 @@ def test_gemm_random_shapes(pb):
         K = int(rng.integers(1, 12)) * 64
         epi = int(rng.integers(0, 3))
         tile = [0, 64, 128, 256, 384][case % 5]
-        if tile == 384 and elt == F32:
+        if tile in (384, 192, 385) and elt == F32:
             tile = 0
         print("gemm sweep", case, elt, M, N, K, epi, tile, flush=True)
         X = rng.standard_normal((M, K)).astype(np.float32)
@@ -578,7 +585,9 @@ LN_NO_RESIDUAL = 16
 
 @pytest.mark.parametrize("elt,M,N,K,tile,splits", [
     (BF16, 600, 1024, 1024, 256, 1), (BF16, 333, 768, 3072, 256, 1), (BF16, 600, 1024, 1024, 384, 1),
-    (BF16, 257, 520, 256, 384, 1), (BF16, 300, 768, 768, 128, 1), (BF16, 100, 264, 192, 64, 1), (BF16, 77, 1024, 4096, 0, 1),
+    (BF16, 257, 520, 256, 384, 1), (BF16, 600, 1024, 1024, 385, 1), (BF16, 257, 520, 256, 385, 1), (BF16, 1600, 1024, 4096, 385, 1),
+    (BF16, 600, 1024, 1024, 192, 1), (BF16, 257, 520, 256, 192, 1), (BF16, 200, 1024, 4096, 192, 8),
+    (BF16, 1600, 1024, 1024, 192, 4), (BF16, 130, 768, 192, 192, 3), (BF16, 300, 768, 768, 128, 1), (BF16, 100, 264, 192, 64, 1), (BF16, 77, 1024, 4096, 0, 1),
     (F32, 300, 768, 768, 128, 1), (F32, 100, 264, 96, 64, 1), (F32, 513, 1024, 1024, 0, 1),
     (BF16, 200, 1024, 4096, 128, 4), (BF16, 64, 768, 768, 64, 3), (F32, 200, 1024, 1024, 64, 2),
 ])
