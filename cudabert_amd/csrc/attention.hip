@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void attention_kernel(
     const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
     const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
     unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale, int ctx_packed,
-    const int* __restrict__ cu) {
+    const int* __restrict__ cu, int first_only) {
     constexpr int ES = (ELT == kBF16) ? 2 : 4;
     constexpr int ROWB = 64 * ES;            // bytes per Q/K row
     constexpr int KK = ROWB / 32;            // MFMA k-steps over the head dim (4 bf16 / 8 f32)
@@ -46,8 +46,9 @@ __global__ __launch_bounds__(256) void attention_kernel(
     const int q0 = (blockIdx.x * 4 + wave) * 32;
     // compact rows: only queries below the sequence's length exist, at rows cu[b] + query
     const int qlen = cu ? cu[b + 1] - cu[b] : S;
-    const size_t row_base = cu ? (size_t)cu[b] : (size_t)b * S;
-    if (q0 >= qlen) return;                   // whole wave leaves; no barriers below
+    // first_only: only query 0 of every sequence is wanted, as row b of a [B, hidden] context
+    const size_t row_base = first_only ? (size_t)b : cu ? (size_t)cu[b] : (size_t)b * S;
+    if (q0 >= qlen || (first_only && q0 != 0)) return;      // whole wave leaves; no barriers below
 
     const size_t bh = (size_t)b * heads + h;
     const unsigned char* qb = q + bh * S * ROWB;
@@ -167,7 +168,7 @@ __global__ __launch_bounds__(256) void attention_kernel(
 
     // ---- normalise and store: lane owns query q0 + l32, features 32 db + 8 j + 4 g + e ----
     const int qi = q0 + l32;
-    if (qi >= qlen) return;
+    if (qi >= qlen || (first_only && qi != 0)) return;
     const float inv = 1.0f / run_sum;
     const size_t hidden = (size_t)heads * 64;
     unsigned char* orow = ctx + ((row_base + qi) * hidden + (size_t)h * 64) * ES;
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
     const unsigned char* __restrict__ vt, const float* __restrict__ maskadd,
     unsigned char* __restrict__ ctx, int heads, int S, int Sp, int vstride, float scale_log2e, int ctx_packed,
-    const int* __restrict__ cu) {
+    const int* __restrict__ cu, int first_only) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char* sK = smem;
     unsigned char* sV = smem + (size_t)Sp * 128;
@@ -305,8 +306,11 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const int q0 = wave * 32;
     // compact rows: only queries below the sequence's length exist, at rows cu[b] + query
     const int qlen = cu ? cu[b + 1] - cu[b] : S;
-    const size_t row_base = cu ? (size_t)cu[b] : (size_t)b * S;
-    if (q0 >= qlen) return;                   // past the last barrier: a whole wave may leave
+    // first_only: only query 0 of every sequence is wanted, as row b of a [B, hidden] context.  Wave 0 still works on
+    // its 32 queries (a query's bits depend on when its wave moves the reference exponent, i.e. on its wave mates)
+    // and stores one of them.
+    const size_t row_base = first_only ? (size_t)b : cu ? (size_t)cu[b] : (size_t)b * S;
+    if (q0 >= qlen || (first_only && wave != 0)) return;      // past the last barrier: a whole wave may leave
     int qrow = q0 + l32;
     qrow = qrow < qlen ? qrow : qlen - 1;
     uint4 qf[4];
@@ -431,7 +435,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 
     // ---- normalise and store: lane owns query q0 + l32, features 32 db + 8 j + 4 g + e ----
     const int qi = q0 + l32;
-    if (qi >= qlen) return;
+    if (qi >= qlen || (first_only && qi != 0)) return;
     const float inv = 1.0f / run_sum;
     const size_t hidden = (size_t)heads * 64;
     unsigned char* orow = ctx + ((row_base + qi) * hidden + (size_t)h * 64) * 2;
@@ -453,7 +457,8 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
 
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
                       bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream,
-                      const int* cu, bool v_rowmajor) {
+                      const int* cu, bool v_rowmajor, bool first_only) {
+    const int fo = first_only ? 1 : 0;
     if (ctx_packed && elt != kBF16) { set_error("attention: only a bf16 context can be packed"); return false; }
     const int cp = ctx_packed ? 1 : 0;
     if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
@@ -492,19 +497,19 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
         }
         if (v_rowmajor)
             hipLaunchKernelGGL(attention_lds_kernel<true>, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd,
-                               cc, heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);
+                               cc, heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu, fo);
         else
             hipLaunchKernelGGL(attention_lds_kernel<false>, dim3(heads, B), dim3(2 * Sp), lds, stream, qc, kc, vc, maskadd,
-                               cc, heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu);
+                               cc, heads, S, Sp, vstride, scale * 1.4426950408889634f, cp, cu, fo);
         CUBERT_HIP_OK(hipGetLastError());
         return true;
     }
     if (v_rowmajor) { set_error("attention: a row-major V needs bf16 operands and S <= 512"); return false; }
-    dim3 grid((S + 127) / 128, heads, B), block(256);
+    dim3 grid(first_only ? 1 : (S + 127) / 128, heads, B), block(256);
     if (elt == kBF16)
-        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu);
+        hipLaunchKernelGGL(attention_kernel<kBF16>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu, fo);
     else
-        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu);
+        hipLaunchKernelGGL(attention_kernel<kF32>, grid, block, 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp, scale, cp, cu, fo);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }

@@ -62,6 +62,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.fuse_residual = env_int("CUBERT_FUSE_RESIDUAL", 1) != 0;
     opt.fuse_layernorm = env_int("CUBERT_FUSE_LAYERNORM", 1) != 0;
     opt.v_rowmajor = env_int("CUBERT_V_ROWMAJOR", 1) != 0;
+    opt.first_token_last_layer = env_int("CUBERT_FIRST_TOKEN_LAST_LAYER", 1) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
     opt.max_seq = maxS;

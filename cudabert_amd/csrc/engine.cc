@@ -200,6 +200,9 @@ bool Model::init(const ModelOptions& opt_in) {
     const size_t o_meta = aa.take(meta_ints * 4), o_seqpad = aa.take(N * H * 4);
     ln_ws_bytes_ = (gemm_ln_workspace_bytes(N) + 255) / 256 * 256;
     const size_t o_lnws = aa.take(ln_ws_bytes_ * kMaxParts);
+    const size_t NC = (size_t)kMaxParts * 1024;       // first-token rows: B <= 1024 per part, parts 1024 rows apart
+    const size_t o_xc = aa.take(NC * H * 4), o_yc = aa.take(NC * H * 4), o_xbc = elt == kBF16 ? aa.take(NC * H * 2) : 0;
+    const size_t o_ctxc = aa.take(NC * H * es), o_hc = aa.take(NC * I * es);
     act_bytes_ = aa.off;
     size_t free_b = 0, total_b = 0;
     CUBERT_HIP_OK(hipMemGetInfo(&free_b, &total_b));
@@ -223,6 +226,11 @@ bool Model::init(const ModelOptions& opt_in) {
     d_meta_ = reinterpret_cast<int*>(ablock_ + o_meta);
     seqpad_ = reinterpret_cast<float*>(ablock_ + o_seqpad);
     ln_ws_ = ablock_ + o_lnws;       // all zero from the clearing above, which is what the first launch needs
+    xc32_ = reinterpret_cast<float*>(ablock_ + o_xc);
+    yc32_ = reinterpret_cast<float*>(ablock_ + o_yc);
+    xbc_ = elt == kBF16 ? reinterpret_cast<bf16_t*>(ablock_ + o_xbc) : nullptr;
+    ctxc_ = ablock_ + o_ctxc;
+    hc_ = ablock_ + o_hc;
     CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_meta_), meta_ints * 4, hipHostMallocDefault));
     CUBERT_HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&h_in_), 3 * N * 4, hipHostMallocDefault));
     CUBERT_HIP_OK(hipStreamSynchronize(stream_));
@@ -284,6 +292,8 @@ bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B,
     // the caller cannot see the sequence output, the batch is too large for hipGraph replay and at
     // least 5 % of it is padding.
     const bool too_big_for_graph = opt_.graph_max_tokens <= 0 || (long)n > opt_.graph_max_tokens;
+    // The caller will not see the sequence output: the last layer only has to produce what the pooler reads.
+    first_only_ = !need_seq && opt_.first_token_last_layer;
     if (mask && (opt_.varlen == 1 || (opt_.varlen < 0 && !need_seq && too_big_for_graph))) {
         std::vector<int> lens(B);
         bool prefix = true;
@@ -304,6 +314,7 @@ bool Model::forward_host(const int* ids, const int* seg, const int* mask, int B,
 
 bool Model::forward_device_lens(const int* d_ids, const int* d_seg, const int* h_lens, int B, int S) {
     if (!check_shape(B, S)) return false;
+    first_only_ = false;
     if (!d_ids || !d_seg || !h_lens) { set_error("input_ids, token_type_ids and lengths must not be null"); return false; }
     for (int b = 0; b < B; ++b)
         if (h_lens[b] < 1 || h_lens[b] > S) {
@@ -379,6 +390,7 @@ bool Model::run_compact(const int* lens, int B, int S) {
 
 bool Model::forward_device(const int* d_ids, const int* d_seg, const int* d_mask, int B, int S) {
     if (!check_shape(B, S)) return false;
+    first_only_ = false;
     if (!d_ids || !d_seg) { set_error("input_ids and token_type_ids must not be null"); return false; }
     const size_t n = (size_t)B * S, cap = (size_t)cap_tokens_;
     CUBERT_HIP_OK(hipMemcpyAsync(d_in_, d_ids, n * 4, hipMemcpyDeviceToDevice, stream_));
@@ -395,8 +407,9 @@ bool Model::run(int B, int S, bool has_mask) {
     last_classified_ = false;
     const long tokens = (long)B * S;
     if (opt_.graph_max_tokens <= 0 || tokens > opt_.graph_max_tokens) return enqueue(B, S, has_mask);
-    // One entry per (B, S, mask) shape; the key is injective for every B <= 1024 and any S.
-    const unsigned long long key = ((unsigned long long)B << 33) | ((unsigned long long)(unsigned)S << 1) | (has_mask ? 1ull : 0ull);
+    // One entry per (B, S, mask, kind of last layer) shape; the key is injective for every B <= 1024 and any S.
+    const unsigned long long key = ((unsigned long long)B << 33) | ((unsigned long long)(unsigned)S << 1) | (has_mask ? 1ull : 0ull) |
+                                   (first_only_ ? 1ull << 62 : 0ull);
     auto it = graphs_.find(key);
     if (it != graphs_.end() && it->second.exec) {
         it->second.last_use = ++graph_clock_;
@@ -562,7 +575,43 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
         g.rowmap = cp ? cp->rowmap : nullptr;
         g.x_packed = g.w_packed = pk;
         if (!mark(kPhQKV) || !launch_gemm(g, st)) return false;
+        // The last layer of a pass whose caller gets no sequence output: keys and values are needed of every token,
+        // everything after them only of the first token of each sequence, which is all the pooler reads.  Its B rows
+        // go through the same kernels as row b * S of the full pass would (K is never split for them, and every
+        // kernel treats a row the same whatever else is in the launch), so the pooled output keeps its bits.
+        const bool first = first_only_ && i == D.layers - 1 && sp_ao == 1 && sp_fo == 1;
         if (!mark(kPhAttention)) return false;
+        if (first) {
+            const size_t c0 = (size_t)part * 1024;
+            float* xc = xc32_ + c0 * H;
+            float* yc = yc32_ + c0 * H;
+            bf16_t* xbc = xbc_ ? xbc_ + c0 * H : nullptr;
+            unsigned char* ctxc = static_cast<unsigned char*>(ctxc_) + c0 * H * es;
+            unsigned char* hc = static_cast<unsigned char*>(hc_) + c0 * I * es;
+            const void* xcin = elt == kBF16 ? static_cast<const void*>(xbc) : static_cast<const void*>(xc);
+            if (!launch_attention(q, k, vt, maskadd, ctxc, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow, true)) return false;
+            if (!launch_gather_first_rows(x32, cu, xc, B, S, H, st)) return false;
+            g = GemmParams();
+            g.elt = elt; g.out_elt = kF32; g.X = ctxc; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = yc;
+            g.M = B; g.N = H; g.K = H; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
+            g.residual = fuse_res ? xc : nullptr;
+            if (!mark(kPhAttnOut) || !launch_gemm(g, st)) return false;
+            if (!mark(kPhLayerNorm)) return false;
+            if (!launch_add_layernorm(xc, yc, kF32, L.g1, L.be1, xbc, pk, B, H, st, 1, !fuse_res)) return false;
+            g = GemmParams();
+            g.elt = elt; g.out_elt = elt; g.X = xcin; g.ldx = H; g.W = L.w_in; g.bias = L.b_in; g.Y = hc;
+            g.M = B; g.N = I; g.K = H; g.epilogue = kEpiBiasGelu; g.x_packed = g.w_packed = g.y_packed = pk;
+            if (!mark(kPhFFNIn) || !launch_gemm(g, st)) return false;
+            g = GemmParams();
+            g.elt = elt; g.out_elt = kF32; g.X = hc; g.ldx = I; g.W = L.w_out; g.bias = L.b_out; g.Y = yc;
+            g.M = B; g.N = H; g.K = I; g.epilogue = kEpiBias; g.x_packed = g.w_packed = pk;
+            g.residual = fuse_res ? xc : nullptr;
+            if (!mark(kPhFFNOut) || !launch_gemm(g, st)) return false;
+            if (!mark(kPhLayerNorm)) return false;
+            if (!launch_add_layernorm(xc, yc, kF32, L.g2, L.be2, nullptr, false, B, H, st, 1, !fuse_res)) return false;
+            if (!mark(kPhPooler)) return false;
+            return launch_pooler(xc, w_pool_, elt, b_pool_, pooled_ + (size_t)b0 * H, B, 1, H, st, nullptr);
+        }
         if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
@@ -619,6 +668,7 @@ bool Model::profile_device(const int* d_ids, const int* d_seg, const int* d_mask
     if (d_mask) CUBERT_HIP_OK(hipMemcpyAsync(d_in_ + 2 * cap, d_mask, n * 4, hipMemcpyDeviceToDevice, stream_));
     B_ = B;
     S_ = S;
+    first_only_ = false;
     last_compact_ = false;
     last_has_mask_ = d_mask != nullptr;
     last_classified_ = false;

@@ -34,6 +34,8 @@ struct ModelOptions {
     int varlen = -1;               // host-input calls with prefix masks compute only the valid tokens: 1 always,
                                    // 0 never, -1 when the caller asks for no sequence output (see forward_host)
     int graph_max_tokens = 8192;   // capture a hipGraph for batches up to this many tokens (0: never)
+    bool first_token_last_layer = true;   // calls that hand back no sequence output compute the last layer for the first
+                                          // token of every sequence only (everything the pooler reads)
     int graph_cache = 64;          // instantiated hipGraphs kept per model (least recently used is dropped)
     std::string dir;
 };
@@ -139,6 +141,11 @@ class Model {
     bool recovered_ = false;           // the last sync() repeated the pass: copies enqueued before it carry the discarded results
     bool last_has_mask_ = false, last_classified_ = false;
     std::vector<int> last_lens_;       // lengths of the last unpadded pass
+    // Last layer for the first tokens only: [kMaxParts * 1024] rows each (a part's sequences at part * 1024)
+    float *xc32_ = nullptr, *yc32_ = nullptr;      // residual stream / GEMM result of those rows
+    bf16_t* xbc_ = nullptr;                        // bf16 copy (bf16 mode)
+    void *ctxc_ = nullptr, *hc_ = nullptr;         // attention context / FFN activation of those rows
+    bool first_only_ = false;                      // the pass being enqueued (and the last one run) is of that kind
     bool last_compact_ = false;
     int cur_parts_ = 1;          // parts of the pass being enqueued
     int B_ = 0, S_ = 0;

@@ -111,8 +111,10 @@ bool gemm_ln_supported(int M, int N, int K, int elt);
 // ctx_packed (bf16 only): write ctx in the packed GEMM-operand layout (common.h).
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd,
                       void* ctx, bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt,
-                      hipStream_t stream, const int* cu = nullptr, bool v_rowmajor = false);
+                      hipStream_t stream, const int* cu = nullptr, bool v_rowmajor = false, bool first_only = false);
 // v_rowmajor (bf16, S <= 512 only): `vt` holds V as [B, heads, S, 64] like k.
+// first_only: only the context of every sequence's first token is produced, as row b of ctx [B, heads*64] (same bits
+// as row b * S of the full result).
 
 // ----------------------------------------------------------- LayerNorm -----
 // x <- LayerNorm(x + y) * gamma + beta   over rows of length H, in place on the
@@ -158,6 +160,10 @@ bool launch_classifier(const float* pooled, const float* kernel, const float* bi
 // the pooler op_Linear of cuda_bert/utils/bert.cu:238-247; modeling.py:347-353).
 bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, float* pooled, int B, int S, int H,
                    hipStream_t stream, const int* cu = nullptr);
+
+// out[b, :] = x[first row of sequence b, :] (row b * S, or cu[b] on compact rows): the residual rows of a last
+// layer that is only computed for the first tokens.
+bool launch_gather_first_rows(const float* x, const int* cu, float* out, int B, int S, int H, hipStream_t stream);
 
 // Compact rows -> padded [B, S, H] float32 (zeros on the positions past a sequence's length).
 bool launch_unpad_rows(const float* xc, const int* cu, float* out, int B, int S, int H, hipStream_t stream);

@@ -514,6 +514,17 @@ __global__ __launch_bounds__(256) void unpad_rows_kernel(const float* __restrict
     }
 }
 
+// out[b, :] = x[first row of sequence b, :]; one wave per sequence.
+__global__ __launch_bounds__(256) void gather_first_rows_kernel(const float* __restrict__ x, const int* __restrict__ cu,
+                                                                float* __restrict__ out, int B, int S, int H) {
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= B) return;
+    const float* src = x + (cu ? (size_t)cu[b] : (size_t)b * S) * H;
+    for (int i = lane * 4; i < H; i += 256)
+        *reinterpret_cast<f32x4_t*>(out + (size_t)b * H + i) = *reinterpret_cast<const f32x4_t*>(src + i);
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
@@ -642,6 +653,16 @@ bool launch_pooler(const float* x, const void* W, int w_elt, const float* bias, 
     if (w_elt == kBF16) hipLaunchKernelGGL(pooler_kernel<kBF16>, grid, block, 0, stream, x, wc, bias, pooled, S, H, cu);
     else if (w_elt == kF32) hipLaunchKernelGGL(pooler_kernel<kF32>, grid, block, 0, stream, x, wc, bias, pooled, S, H, cu);
     else { set_error("pooler: bad weight type"); return false; }
+    CUBERT_HIP_OK(hipGetLastError());
+    return true;
+}
+
+bool launch_gather_first_rows(const float* x, const int* cu, float* out, int B, int S, int H, hipStream_t stream) {
+    if (!x || !out || B <= 0 || S <= 0 || H <= 0 || H % 4 != 0 || !aligned16(x) || !aligned16(out)) {
+        set_error("gather: bad arguments");
+        return false;
+    }
+    hipLaunchKernelGGL(gather_first_rows_kernel, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, stream, x, cu, out, B, S, H);
     CUBERT_HIP_OK(hipGetLastError());
     return true;
 }

@@ -52,7 +52,11 @@ void release_model(void* model);
  * prints the reason to stderr and terminates the process with
  * exit(EXIT_FAILURE), which is what the reference does through its asserts
  * and checkCudaErrors (cuda_bert/utils/manager.cu:100-108, common.h:58-65).
- * Callers that want an error code use cubert_encode instead. */
+ * Callers that want an error code use cubert_encode instead.
+ * Since the caller receives only [B, hidden], the last encoder layer is computed for the first token of every
+ * sequence only (keys and values still of every token): the pooled output has the bits of the full pass, the
+ * device-side sequence buffer (cubert_seq_ptr) is not defined after such a call.  The same holds for
+ * Cuda_Classify and cubert_encode with seq_out == NULL; CUBERT_FIRST_TOKEN_LAST_LAYER=0 at init turns it off. */
 void Cuda_Bert(void* model, float* output, int* words, int* token_types, int batchsize,
                int seq_length, int* attention_mask);
 

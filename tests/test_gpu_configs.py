@@ -76,8 +76,11 @@ def test_cfg1_base_b128_s128_full_batch(pb, base_ckpt, precision):
     m = load(pb, W.BASE, base_ckpt.dir(exact), precision, B, S)
     try:
         pooled, seq, cls = pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)
+        probs_only = np.zeros((B, 2), np.float32)           # pooled-only call (last layer for the first tokens only)
+        pb.classify(m, probs_only, ids, seg, B, S, 2, mask)
     finally:
         pb.unload_model(m)
+    assert np.array_equal(probs_only, cls)
     n = 4
     npy = base_ckpt.npy(exact)
     seq_ref, pooled_ref = O.forward_torch(npy, W.BASE.heads, ids[:n], seg[:n], mask[:n])
@@ -123,8 +126,12 @@ def test_bf16_mode_on_an_unrounded_fp32_checkpoint(pb, base_ckpt, large_ckpt, wh
     m = load(pb, D, ck.raw, BF16, B, S)
     try:
         pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+        pooled_only = np.ones((B, D.hidden), np.float32)    # Cuda_Bert on the same batch (cfg2: two stream parts, unpadded)
+        pb.bert(m, pooled_only, ids, seg, B, S, mask)
     finally:
         pb.unload_model(m)
+    if which == "large":        # (the short batch of configuration 0 splits K by its row count, which differs between the two calls)
+        assert np.array_equal(pooled_only, pooled)
     seq_ref, pooled_ref = O.forward_torch(ck.npy_raw, D.heads, ids[:n], seg[:n], mask[:n])
     e_seq, e_pool = err(seq[:n], seq_ref), err(pooled[:n], pooled_ref)
     rms = float(np.sqrt(np.mean((seq[:n] - seq_ref) ** 2)))
@@ -283,8 +290,12 @@ def test_cfg4_large_b64_s512_skewed(pb, large_ckpt):
         torch.cuda.synchronize()
         pb.check(pb.lib.cubert_forward_device_lens(m, d[0].data_ptr(), d[1].data_ptr(), lens.ctypes.data, B, S))
         pooled_u, seq_u = device_results(pb, m, B, S, D.hidden)
+        # pooled-only host call: valid tokens only, last layer for the first tokens only -- the same bits
+        pooled_only = np.ones((B, D.hidden), np.float32)
+        pb.bert(m, pooled_only, ids, seg, B, S, mask)
     finally:
         pb.unload_model(m)
+    assert np.array_equal(pooled_only, pooled)
     assert np.isfinite(seq).all() and np.allclose(cls.sum(1), 1.0, atol=1e-5)
     assert np.array_equal(pooled_p, pooled[perm]) and np.array_equal(seq_p, seq[perm])
     valid = mask.astype(bool)
@@ -344,6 +355,7 @@ def test_pooled_only_host_calls_compute_valid_tokens_only(pb, tmp_path, monkeypa
     ids, seg, mask = synth.make_inputs(B, S, [40, 3, 17, 1, 22], vocab=D.vocab, seed=3, prune=False)
     seq_ref, pooled_ref = O.forward_torch(npy, D.heads, ids, seg, mask)
     monkeypatch.setenv("CUBERT_SPLIT_K", "0")      # split K would group the sums by the row count
+    monkeypatch.setenv("CUBERT_FIRST_TOKEN_LAST_LAYER", "0")     # this test reads the sequence buffer such calls leave behind
     for precision in (F32, BF16):
         m = load(pb, D, wdir, precision, B, S)
         try:
@@ -367,6 +379,49 @@ def test_pooled_only_host_calls_compute_valid_tokens_only(pb, tmp_path, monkeypa
             assert (seq_dev[~valid] != 0).any()
         finally:
             pb.unload_model(m)
+
+
+@pytest.mark.parametrize("precision", [F32, BF16])
+def test_pooled_only_calls_compute_the_last_layer_for_first_tokens_only(pb, tmp_path, monkeypatch, precision):
+    """Cuda_Bert / Cuda_Classify / cubert_encode(seq_out = NULL) hand back [B, hidden] (cuda_bert/cuda_bert.cu:55-70):
+    after the last layer's keys and values only the first token of every sequence matters.  Those B rows run through
+    the same kernels as row b * S of the full pass, so the results are the full pass's bit for bit: padded pass,
+    unpadded pass, eager and replayed from a graph, one stream and two."""
+    D = W.TINY
+    state = W.bf16_representable(W.synth_state(D, seed=22, degenerate=False))
+    wdir = W.export_npy_dir(state, str(tmp_path / "w"))
+    B, S = 6, 40
+    ids, seg, mask = synth.make_inputs(B, S, [40, 3, 17, 1, 22, 40], vocab=D.vocab, seed=4, prune=False)
+    monkeypatch.setenv("CUBERT_SPLIT_K", "0")      # split K would group the sums by the row count
+    monkeypatch.setenv("CUBERT_FIRST_TOKEN_LAST_LAYER", "0")
+    m = load(pb, D, wdir, precision, B, S)
+    try:
+        pooled_full, _, cls_full = pb.encode(m, ids, seg, mask, want_seq=True, want_cls=True)
+    finally:
+        pb.unload_model(m)
+    monkeypatch.delenv("CUBERT_FIRST_TOKEN_LAST_LAYER")
+    for varlen in ("0", "1"):
+        for split_min, graph in (("0", 0), ("1", 0), ("0", 4096), ("1", 4096)):
+            monkeypatch.setenv("CUBERT_VARLEN", varlen)
+            monkeypatch.setenv("CUBERT_SPLIT_MIN_TOKENS", split_min)
+            m = load(pb, D, wdir, precision, B, S, graph=graph)
+            try:
+                for rep in range(3 if graph else 1):
+                    out = np.ones((B, D.hidden), np.float32)
+                    pb.bert(m, out, ids, seg, B, S, mask)
+                    assert np.array_equal(out, pooled_full), (varlen, split_min, graph, rep)
+                    probs = np.zeros((B, 2), np.float32)
+                    pb.classify(m, probs, ids, seg, B, S, 2, mask)
+                    assert np.array_equal(probs, cls_full)
+                    # a call that wants the sequence output in between gets the full pass
+                    pooled2, seq2, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+                    assert np.array_equal(pooled2, pooled_full) and np.isfinite(seq2).all()
+                # no mask at all: every position valid
+                out2, _, _ = pb.encode(m, ids, seg, None)          # seq_out == NULL: a pooled-only call
+                pooled3, _, _ = pb.encode(m, ids, seg, None, want_seq=True)
+                assert np.array_equal(out2, pooled3)
+            finally:
+                pb.unload_model(m)
 
 
 # ------------------------------------------------------------------ hipGraph cache ----
