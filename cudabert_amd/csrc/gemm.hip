@@ -225,6 +225,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
         CUBERT_ISSUE_TILE(lds1, kt0 + 1);
         CUBERT_ISSUE_TILE(lds2, kt0 + 2);
     }
+    // The four-stage kernel runs launches of a few workgroups and a few K steps each, i.e. chains of round trips:
+    // what the epilogue adds (bias, first residual rows) is requested now, behind the first tiles.
+    constexpr bool SPLITK = (EPI == kEpiBias || EPI == kEpiBiasRes) && OUT == kF32;      // the only combinations launch_gemm splits
+    constexpr bool PREFETCH = NS == 4 && BT == 64;
+    f32x4_t bias[4 * NB];
+    EpiPrefetch<EpiGeometry<OUT, EPI, NB, SPLITK, 4>::PB> pre;
+    if constexpr (PREFETCH) {
+        if constexpr (gemm_bias_at_readout<OUT, EPI>()) gemm_epilogue_prefetch<OUT, EPI, NB, SPLITK, 4>(p, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, &pre);
+        else gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
+    }
     __builtin_amdgcn_s_waitcnt(WAIT_IMM);
     if constexpr (NS == 4) __builtin_amdgcn_s_barrier();
     else __syncthreads();
@@ -249,11 +259,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmDev p) {
 #undef CUBERT_FENCE_FRAGS
 #undef CUBERT_K_STEP
 
-    f32x4_t bias[4 * NB];      // fetched here rather than before the loop: no registers to spare there
-    constexpr bool SPLITK = (EPI == kEpiBias || EPI == kEpiBiasRes) && OUT == kF32;      // the only combinations launch_gemm splits
-    if constexpr (!gemm_bias_at_readout<OUT, EPI>()) gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
+    // (the larger tiles fetch their bias here rather than before the loop: no registers to spare there)
+    if constexpr (!PREFETCH && !gemm_bias_at_readout<OUT, EPI>()) gemm_load_bias<NB, SPLITK>(p, n0 + wn * (BT / 2), g, bias);
     // every wave is past the last step's barrier: the tiles are dead, lds0 is free for staging
-    gemm_epilogue<OUT, EPI, NB, NB, SPLITK, 4, true>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64));
+    gemm_epilogue<OUT, EPI, NB, NB, SPLITK, 4, true>(p, acc, bias, n0 + wn * (BT / 2), m0 + wm * (BT / 2), l32, g, lds0 + wave * (BT * 64),
+                                                     PREFETCH && gemm_bias_at_readout<OUT, EPI>() ? &pre : nullptr);
 }
 
 template <int ELT, int OUT, int EPI, int BT, int NS = 2>

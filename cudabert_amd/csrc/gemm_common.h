@@ -192,9 +192,54 @@ __device__ __forceinline__ void gemm_load_bias(const GemmDev& p, int n_base, int
 // layout of the stores (whole row segments).  The fetches go out RPB read-out steps at a time; with RDB
 // the next batch is requested before the current one is consumed (two batches of registers), which a
 // kernel with one workgroup per CU needs because nothing else covers the latency there.
+// What the read-out phase of a float32 epilogue adds to the first rows it handles: the bias quad of the lane's features
+// and (kEpiBiasRes) the first batch of residual rows.  gemm_epilogue fetches them itself; a kernel whose launch is too
+// short to hide that round trip behind anything else (a few K steps per workgroup) asks for them before its K loop
+// with gemm_epilogue_prefetch and hands them in.
+template <int PB>
+struct EpiPrefetch {
+    f32x4_t bias_ro;
+    f32x4_t res0[PB];
+};
+
+template <int OUT, int EPI, int NBI, bool SPLITK = false, int RPB = 4>
+struct EpiGeometry {
+    static constexpr int OES = (OUT == kBF16) ? 2 : 4;
+    static constexpr int RB = 32 * NBI * OES;      // bytes per token row of the staging block
+    static constexpr int CH = RB / 16;             // 16-byte chunks per row
+    static constexpr int RPI = 64 / CH;            // rows one store instruction covers
+    static constexpr int EPC = 16 / OES;           // elements per chunk
+    static constexpr bool RES = EPI == kEpiBiasRes;
+    static constexpr int NIT = 32 / RPI;                               // read-out steps per block column
+    static constexpr int PB = RES ? (NIT < RPB ? NIT : RPB) : NIT;     // steps per residual batch
+};
+
+template <int OUT, int EPI, int NBI, bool SPLITK = false, int RPB = 4>
+__device__ __forceinline__ void gemm_epilogue_prefetch(const GemmDev& p, int n_base, int m_base, int l32, int g,
+                                                       EpiPrefetch<EpiGeometry<OUT, EPI, NBI, SPLITK, RPB>::PB>* pre) {
+    typedef EpiGeometry<OUT, EPI, NBI, SPLITK, RPB> G;
+    static_assert(gemm_bias_at_readout<OUT, EPI>(), "only float32 results take their bias in the read-out phase");
+    const int lane = l32 + 32 * g;
+    const int rrow = lane / G::CH, rc = lane % G::CH;
+    bool first = true;
+    if constexpr (SPLITK) first = blockIdx.y == 0;          // split K: bias and residual are added once
+    const int n = n_base + rc * G::EPC;
+    pre->bias_ro = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    if (first) pre->bias_ro = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
+    if constexpr (G::RES) {
+#pragma unroll
+        for (int s = 0; s < G::PB; ++s) {
+            const int mm = m_base + s * G::RPI + rrow;
+            pre->res0[s] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            if (first) pre->res0[s] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p.R + (size_t)(mm < p.M ? mm : p.M - 1) * p.N + (n < p.N ? n : p.N - 4)));
+        }
+    }
+}
+
 template <int OUT, int EPI, int NBI, int NBJ, bool SPLITK = false, int RPB = 4, bool RDB = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[NBI][NBJ], const f32x4_t (&bias)[4 * NBI],
-                                              int n_base, int m_base, int l32, int g, unsigned char* scratch) {
+                                              int n_base, int m_base, int l32, int g, unsigned char* scratch,
+                                              const EpiPrefetch<EpiGeometry<OUT, EPI, NBI, SPLITK, RPB>::PB>* pre = nullptr) {
     constexpr int OES = (OUT == kBF16) ? 2 : 4;
     constexpr int RB = 32 * NBI * OES;      // bytes per token row of the staging block
     constexpr int CH = RB / 16;             // 16-byte chunks per row
@@ -219,15 +264,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev& p, f32x16_t (&acc)[
             r[s] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p.R + (size_t)(mm < p.M ? mm : p.M - 1) * p.N + (n < p.N ? n : p.N - 4)));
         }
     };
-    if constexpr (RES && RDB)
-        if (addres) fetch_res(0, 0, res[0]);
+    if constexpr (RES && RDB) {
+        if (pre) {
+#pragma unroll
+            for (int s = 0; s < PB; ++s) res[0][s] = pre->res0[s];
+        } else if (addres) {
+            fetch_res(0, 0, res[0]);
+        }
+    }
     constexpr bool BIAS_RO = gemm_bias_at_readout<OUT, EPI>();
     f32x4_t bias_ro = {0.0f, 0.0f, 0.0f, 0.0f};
     if constexpr (BIAS_RO) {
         bool addb = true;
         if constexpr (SPLITK) addb = blockIdx.y == 0;           // split K: the bias is added once
         const int n = n_base + rc * EPC;
-        if (addb) bias_ro = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
+        if (pre) bias_ro = pre->bias_ro;
+        else if (addb) bias_ro = *reinterpret_cast<const f32x4_t*>(p.bias + (n < p.N ? n : p.N - 4));
     }
     // compact rows: the token of this lane's row in every block row, fetched together up front;
     // the read-out phase takes a row's token from the lane that owns it

@@ -24,38 +24,18 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// Normalises the row held in v[][] (lane owns elements c*256 + lane*4 + e) and
-// writes it to x (f32) and optionally xb (bf16).
-// xb (optional) receives the bf16 copy: row-major when xb_packed == 0, else in
-// the packed GEMM-operand layout (common.h).
-__device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H, int lane,
-                                                const float* __restrict__ gamma,
-                                                const float* __restrict__ beta, float* xrow,
-                                                bf16_t* xb, int row, int xb_packed) {
-    // Row statistics in the engine's canonical order (common.h): chunk c holds the slots 2 c (lanes
-    // 0..31) and 2 c + 1 (lanes 32..63); slots past the row's end hold no features and add nothing.
-    const bool upper = lane >= 32;
-    float ssum[2 * kMaxChunks], sm2[2 * kMaxChunks], scnt[2 * kMaxChunks], sinv[2 * kMaxChunks];
-#pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int left = H - 128 * (2 * c + u);
-            const int cnt = left < 0 ? 0 : (left > 128 ? 128 : left);
-            scnt[2 * c + u] = (float)cnt;
-            sinv[2 * c + u] = cnt > 0 ? 1.0f / (float)cnt : 0.0f;
-        }
-        const bool in = c * 256 + lane * 4 < H;
-        float t, q;
-        ln_slot_stats(in ? v[c][0] : 0.0f, in ? v[c][1] : 0.0f, in ? v[c][2] : 0.0f, in ? v[c][3] : 0.0f, in,
-                      upper ? sinv[2 * c + 1] : sinv[2 * c], &t, &q);
-        // every lane gets both slots' statistics
-        const float t_other = __shfl_xor(t, 32), q_other = __shfl_xor(q, 32);
-        ssum[2 * c] = upper ? t_other : t;
-        sm2[2 * c] = upper ? q_other : q;
-        ssum[2 * c + 1] = upper ? t : t_other;
-        sm2[2 * c + 1] = upper ? q : q_other;
-    }
+// Features of a row of H that fall into 128-feature slot s, and the reciprocal (0 for an empty slot).
+__device__ __forceinline__ void ln_slot_count(int H, int s, float* cnt, float* inv) {
+    const int left = H - 128 * s;
+    const int c = left < 0 ? 0 : (left > 128 ? 128 : left);
+    *cnt = (float)c;
+    *inv = c > 0 ? 1.0f / (float)c : 0.0f;
+}
+
+// Row mean and 1 / sigma from the (sum, M2) of the row's slots, in the engine's canonical order (common.h):
+// slots past the row's end hold no features and add nothing.
+__device__ __forceinline__ void ln_combine_slots(const float (&ssum)[2 * kMaxChunks], const float (&sm2)[2 * kMaxChunks], int H,
+                                                 float* mean_out, float* rstd_out) {
     const float inv_n = 1.0f / (float)H;
     float sum = 0.0f;
 #pragma unroll
@@ -63,25 +43,67 @@ __device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H
     const float mean = ln_row_mean(sum, inv_n);
     float m2 = 0.0f;
 #pragma unroll
-    for (int s = 0; s < 2 * kMaxChunks; ++s)
-        if (128 * s < H) m2 = ln_merge_slot(m2, ssum[s], sm2[s], scnt[s], sinv[s], mean);
-    const float rstd = ln_finalize(m2, inv_n);
+    for (int s = 0; s < 2 * kMaxChunks; ++s) {
+        float cnt, inv;
+        ln_slot_count(H, s, &cnt, &inv);
+        if (128 * s < H) m2 = ln_merge_slot(m2, ssum[s], sm2[s], cnt, inv, mean);
+    }
+    *mean_out = mean;
+    *rstd_out = ln_finalize(m2, inv_n);
+}
+
+// (sum, M2) of the two slots of chunk c (features c * 256 + lane * 4 ..): every lane gets both, lower slot first.
+__device__ __forceinline__ void ln_chunk_stats(const float (&v)[4], int c, int H, int lane, float* sum_lo, float* m2_lo,
+                                               float* sum_hi, float* m2_hi) {
+    const bool upper = lane >= 32;
+    float cnt, inv_lo, inv_hi;
+    ln_slot_count(H, 2 * c, &cnt, &inv_lo);
+    ln_slot_count(H, 2 * c + 1, &cnt, &inv_hi);
+    const bool in = c * 256 + lane * 4 < H;
+    float t, q;
+    ln_slot_stats(in ? v[0] : 0.0f, in ? v[1] : 0.0f, in ? v[2] : 0.0f, in ? v[3] : 0.0f, in, upper ? inv_hi : inv_lo, &t, &q);
+    const float t_other = __shfl_xor(t, 32), q_other = __shfl_xor(q, 32);
+    *sum_lo = upper ? t_other : t;
+    *m2_lo = upper ? q_other : q;
+    *sum_hi = upper ? t : t_other;
+    *m2_hi = upper ? q : q_other;
+}
+
+// Normalises features i .. i + 3 of a row (mean, rstd known) and writes them to x (f32) and optionally to the bf16
+// copy xb: row-major when xb_packed == 0, else in the packed GEMM-operand layout (common.h).
+__device__ __forceinline__ void ln_store4(const float (&v)[4], float mean, float rstd, const f32x4_t& g4, const f32x4_t& b4,
+                                          float* xrow, bf16_t* xb, int row, int i, int H, int xb_packed) {
+    f32x4_t o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = ln_apply(v[e], mean, rstd, g4[e], b4[e]);
+    __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t*>(xrow + i));
+    if (xb) {
+        bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
+        unsigned char* dst = reinterpret_cast<unsigned char*>(xb);
+        const size_t off = xb_packed ? packed_offset(row, i * 2, H * 2 / 64) : ((size_t)row * H + i) * 2;
+        *reinterpret_cast<bf16x4_t*>(dst + off) = ob;
+    }
+}
+
+// Normalises the row held in v[][] (lane owns elements c*256 + lane*4 + e) and
+// writes it to x (f32) and optionally xb (bf16).
+__device__ __forceinline__ void normalise_store(float (&v)[kMaxChunks][4], int H, int lane,
+                                                const float* __restrict__ gamma,
+                                                const float* __restrict__ beta, float* xrow,
+                                                bf16_t* xb, int row, int xb_packed) {
+    float ssum[2 * kMaxChunks], sm2[2 * kMaxChunks];
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c)
+        ln_chunk_stats(v[c], c, H, lane, &ssum[2 * c], &sm2[2 * c], &ssum[2 * c + 1], &sm2[2 * c + 1]);
+    float mean, rstd;
+    ln_combine_slots(ssum, sm2, H, &mean, &rstd);
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
         const int i = c * 256 + lane * 4;
         if (i < H) {
             const f32x4_t g4 = *reinterpret_cast<const f32x4_t*>(gamma + i);
             const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(beta + i);
-            f32x4_t o;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = ln_apply(v[c][e], mean, rstd, g4[e], b4[e]);
-            __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t*>(xrow + i));
-            if (xb) {
-                bf16x4_t ob = {(__bf16)o[0], (__bf16)o[1], (__bf16)o[2], (__bf16)o[3]};
-                unsigned char* dst = reinterpret_cast<unsigned char*>(xb);
-                const size_t off = xb_packed ? packed_offset(row, i * 2, H * 2 / 64) : ((size_t)row * H + i) * 2;
-                *reinterpret_cast<bf16x4_t*>(dst + off) = ob;
-            }
+            ln_store4(v[c], mean, rstd, g4, b4, xrow, xb, row, i, H, xb_packed);
         }
     }
 }
@@ -125,23 +147,30 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
 
 // The same operation for a short batch whose addend comes as the partial sums of a split-K GEMM
 // ([part][rows][H] float32): one workgroup per row, so that the few rows still spread over the
-// chip and every partial sum is requested in one round trip.  Wave w adds up the parts of features
-// 256 w .. 256 w + 255; wave 0 then normalises the row with exactly the arithmetic of
-// add_layernorm_kernel (same per-lane values, same reduction order).
+// chip.  Such a launch is a chain of round trips and little else, so everything it needs -- the row,
+// every partial sum, gamma and beta -- is requested before the first value is used.  Wave w adds up the
+// parts of features 256 w .. 256 w + 255 and forms the statistics of its two slots; the waves exchange
+// those through the LDS, every wave combines them (the same arithmetic in the same order as
+// add_layernorm_kernel, hence the same bits) and normalises its own features.
 __global__ __launch_bounds__(256) void add_layernorm_parts_kernel(float* __restrict__ x, const float* __restrict__ y,
                                                                   const float* __restrict__ gamma,
                                                                   const float* __restrict__ beta,
                                                                   bf16_t* __restrict__ xb, int rows, int H,
                                                                   int xb_packed, int y_parts, int add_x) {
-    __shared__ f32x4_t sums[kMaxChunks][64];
+    __shared__ float stats[kMaxChunks][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int row = blockIdx.x;
     float* xrow = x + (size_t)row * H;
     const int i = wave * 256 + lane * 4;
-    if (i < H) {
+    const bool in = i < H;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4_t g4 = {0.0f, 0.0f, 0.0f, 0.0f}, b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (in) {
         f32x4_t a = {0.0f, 0.0f, 0.0f, 0.0f};
         if (add_x) a = *reinterpret_cast<const f32x4_t*>(xrow + i);
         f32x4_t t = *reinterpret_cast<const f32x4_t*>(y + (size_t)row * H + i);
+        g4 = *reinterpret_cast<const f32x4_t*>(gamma + i);
+        b4 = *reinterpret_cast<const f32x4_t*>(beta + i);
         for (int p0 = 1; p0 < y_parts; p0 += 8) {
             f32x4_t u[8];
 #pragma unroll
@@ -154,20 +183,23 @@ __global__ __launch_bounds__(256) void add_layernorm_parts_kernel(float* __restr
                 if (p0 + j < y_parts) t += u[j];
         }
         a += t;
-        sums[wave][lane] = a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = a[e];
+    }
+    float s_lo, q_lo, s_hi, q_hi;
+    ln_chunk_stats(v, wave, H, lane, &s_lo, &q_lo, &s_hi, &q_hi);
+    if (lane == 0) {
+        stats[wave][0] = s_lo; stats[wave][1] = q_lo; stats[wave][2] = s_hi; stats[wave][3] = q_hi;
     }
     __syncthreads();
-    if (wave != 0) return;
-    float v[kMaxChunks][4];
+    float ssum[2 * kMaxChunks], sm2[2 * kMaxChunks];
 #pragma unroll
     for (int c = 0; c < kMaxChunks; ++c) {
-        if (c * 256 + lane * 4 < H) {
-            const f32x4_t a = sums[c][lane];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[c][e] = a[e];
-        }
+        ssum[2 * c] = stats[c][0]; sm2[2 * c] = stats[c][1]; ssum[2 * c + 1] = stats[c][2]; sm2[2 * c + 1] = stats[c][3];
     }
-    normalise_store(v, H, lane, gamma, beta, xrow, xb, row, xb_packed);
+    float mean, rstd;
+    ln_combine_slots(ssum, sm2, H, &mean, &rstd);
+    if (in) ln_store4(v, mean, rstd, g4, b4, xrow, xb, row, i, H, xb_packed);
 }
 
 __global__ __launch_bounds__(256) void embed_layernorm_kernel(
