@@ -274,21 +274,28 @@ def power_leg(torch, pybert, lib, step, sync, prec, N, I, H):
     rows = (N + 255) // 256 * 256
     bias = torch.zeros(I, device="cuda")
     Y = torch.empty((rows, I), dtype=torch.bfloat16, device="cuda")
-    for name, zero in (("ffn_in_gemm_random_operands", False), ("ffn_in_gemm_zero_operands", True)):
+    # Energy per launch of the FFN-in GEMM (socket power x time): the shipped launch on the pass's kind of data and on
+    # zeros, and variants that move fewer bytes for the same flops -- the 256 x 256 tile (two thirds of the LDS
+    # fragment traffic of the 256 x 128 tile, fewer operand fetches) and other orders of the tiles over the XCDs.
+    variants = (("ffn_in_gemm_random_operands", False, 0, 0), ("ffn_in_gemm_zero_operands", True, 0, 0),
+                ("ffn_in_gemm_tile256x256", False, 256, 0), ("ffn_in_gemm_xcd_contiguous_runs", False, 0, 1 << 16),
+                ("ffn_in_gemm_xcd_4x2", False, 0, 3 << 16), ("ffn_in_gemm_xcd_2x4", False, 0, 5 << 16))
+    for name, zero, tile, pflag in variants:
         X = (torch.zeros if zero else torch.randn)((rows, H), device="cuda").to(torch.bfloat16)
         Wt = ((torch.zeros if zero else torch.randn)((I, H), device="cuda") * 0.02).to(torch.bfloat16)
 
         def launches():
             for _ in range(40):
                 pybert.check(lib.cubert_op_gemm(X.data_ptr(), Wt.data_ptr(), bias.data_ptr(), Y.data_ptr(), N, I, H, H,
-                                                1, 1, 1, 0, 7, st.cuda_stream))
+                                                1, 1, 1, tile, 7 | pflag, st.cuda_stream))
             torch.cuda.synchronize()
-        r = ps.measure(launches, 1.5)
+        r = ps.measure(launches, 1.2)
         if r:
             ms = r.pop("ms_per_call") / 40
             r["avg_launch_ms"] = round(ms, 4)
             r["tflops"] = round(2.0 * N * H * I / ms / 1e9, 1)
             r["frac_mfma_peak"] = round(r["tflops"] / PEAK_TFLOPS["bf16"], 4)
+            r["joules_per_launch"] = round(r["power_w"] * ms / 1e3, 4)
         out[name] = r
     return out
 

@@ -238,6 +238,19 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     const unsigned char* kb = k + bh * S * 128;
     const unsigned char* vb = vt + (VROW ? bh * S * 128 : bh * 64 * (size_t)Sp * 2);
 
+    // Q fragments ("B" operand: column = query), kept for the whole key loop.  Requested first, together with the
+    // K / V loads below: a short batch's launch is one chain of round trips, and this one is then not a link of it.
+    const int q0 = wave * 32;
+    // compact rows: only queries below the sequence's length exist, at rows cu[b] + query
+    const int qlen = cu ? cu[b + 1] - cu[b] : S;
+    uint4 qf[4];
+    {
+        int qrow = q0 + l32;
+        qrow = qrow < qlen ? qrow : qlen - 1;       // qlen >= 1; a wave past the end leaves after the barrier, its loads are harmless
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+            qf[kk] = *reinterpret_cast<const uint4*>(qb + (size_t)qrow * 128 + (2 * kk + g) * 16);
+    }
     // ---- stage K (rows S..Sp-1 zero), V^T and the mask row ----
     // The workgroup has 2 Sp threads, K is 8 Sp and V^T 8 Sp 16-byte chunks: four of each per
     // thread.  All eight loads are issued before the first LDS write so that their latencies
@@ -302,22 +315,11 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
     live = __builtin_amdgcn_readfirstlane(live);
     plain = __builtin_amdgcn_readfirstlane(plain);
 
-    // Q fragments ("B" operand: column = query), kept for the whole key loop.
-    const int q0 = wave * 32;
-    // compact rows: only queries below the sequence's length exist, at rows cu[b] + query
-    const int qlen = cu ? cu[b + 1] - cu[b] : S;
     // first_only: only query 0 of every sequence is wanted, as row b of a [B, hidden] context.  Wave 0 still works on
     // its 32 queries (a query's bits depend on when its wave moves the reference exponent, i.e. on its wave mates)
     // and stores one of them.
     const size_t row_base = first_only ? (size_t)b : cu ? (size_t)cu[b] : (size_t)b * S;
     if (q0 >= qlen || (first_only && wave != 0)) return;      // past the last barrier: a whole wave may leave
-    int qrow = q0 + l32;
-    qrow = qrow < qlen ? qrow : qlen - 1;
-    uint4 qf[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-        qf[kk] = *reinterpret_cast<const uint4*>(qb + (size_t)qrow * 128 + (2 * kk + g) * 16);
-
     f32x16_t o[2];
 #pragma unroll
     for (int db = 0; db < 2; ++db)

@@ -281,6 +281,7 @@ void apply_gemm_flags(cubert::GemmParams* p, int flags) {
     p->y_packed = (flags & CUBERT_Y_PACKED) != 0;
     p->compiler_scheduled = (flags & CUBERT_COMPILER_SCHEDULED) != 0;
     p->splits = CUBERT_SPLITS_OF(flags) > 1 ? CUBERT_SPLITS_OF(flags) : 1;
+    p->xcd_partition = ((flags >> 16) & 0xf) - 1;
 }
 }  // namespace
 

@@ -442,6 +442,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
     const int bk = 128 / es;
     if (p.elt != kBF16 && p.elt != kF32) { set_error("gemm: bad operand type"); return false; }
     if (p.M <= 0 || p.N <= 0 || p.K <= 0) { set_error("gemm: empty problem"); return false; }
+    if (p.xcd_partition != -1 && p.xcd_partition != 0 && p.xcd_partition != 2 && p.xcd_partition != 4) { set_error("gemm: the XCD partition is 0, 2 or 4"); return false; }
     if (p.K % bk != 0) { set_error("gemm: K must be a multiple of " + std::to_string(bk)); return false; }
     if (p.N % 4 != 0) { set_error("gemm: N must be a multiple of 4"); return false; }
     if (p.out_elt == kBF16 && p.N % 8 != 0) { set_error("gemm: N must be a multiple of 8 for bf16 results"); return false; }
@@ -542,6 +543,7 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         d.tiles_n = (p.N + 255) / 256;
         d.tiles_m = (p.M + 127) / 128;
         d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 8);
+        if (p.xcd_partition >= 0) d.xn_parts = p.xcd_partition;
         if (bt == kTile256x128Deep) {
             if (epi == kEpiBiasResLN) { set_error("gemm: the one-per-CU 256x128 tile has no LayerNorm epilogue"); return false; }
             return launch_gemm_bf16_t256x128_deep(d, out, epi, stream);
@@ -553,11 +555,13 @@ bool launch_gemm(const GemmParams& p, hipStream_t stream) {
         d.tiles_n = (p.N + 127) / 128;
         d.tiles_m = (p.M + 127) / 128;
         d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 8);
+        if (p.xcd_partition >= 0) d.xn_parts = p.xcd_partition;
         return launch_gemm_bf16_t128(d, out, epi, stream);
     }
     d.tiles_n = (p.N + bt - 1) / bt;
     d.tiles_m = (p.M + bt - 1) / bt;
     d.xn_parts = gemm_pick_partition((double)p.M * p.K * es, (double)p.N * p.K * es, d.tiles_n, d.tiles_m, 4);
+    if (p.xcd_partition >= 0) d.xn_parts = p.xcd_partition;
     if (p.elt == kBF16) {
         // 256 tile with a multiple of four half-steps: the hand-scheduled kernel
         if (bt == 256 && p.K % 128 == 0 && !p.compiler_scheduled && d.splits == 1)

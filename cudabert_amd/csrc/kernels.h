@@ -83,6 +83,8 @@ struct GemmParams {
     bool compiler_scheduled = false;   // 256 tile: use the generic kernel, not the hand-scheduled one
     // Packed operand layout (common.h): X / W read from it, Y (bf16, plain epilogues) written in it.
     bool x_packed = false, w_packed = false, y_packed = false;
+    int xcd_partition = -1;   // how the eight XCDs divide the tile grid (see tile_of_block): -1 = estimate and choose, 0 = contiguous
+                              // runs of the tile sequence, 2 / 4 = 4 x 2 / 2 x 4 cells (for measurements)
 };
 bool launch_gemm(const GemmParams& p, hipStream_t stream);
 // The tile (a GemmParams::tile value, never 0) and split count launch_gemm's cost model prefers for a problem.

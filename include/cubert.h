@@ -189,6 +189,10 @@ long cubert_capacity_tokens(void* model);
 /* Split K (cubert_op_gemm, epilogue 0, float32 Y): n workgroups share a tile, each reduces 1/n of K
  * and writes its partial sum to Y + i * M * N (the bias is in partial 0); Y holds n * M * N floats and
  * the consumer adds the parts (cubert_op_add_layernorm takes the count in the same flag bits). */
+/* For measurements: how the eight XCDs (each with its own L2) divide the tile grid of a GEMM: n = 0 contiguous runs of the
+ * tile sequence (an XCD owns a band of token rows), 2 or 4: a 4 x 2 / 2 x 4 partition (an XCD keeps half / a quarter of the
+ * weight rows).  Without the flag the library estimates the traffic of each and takes the smallest. */
+#define CUBERT_XCD_PARTITION(n) ((((n) + 1) & 0xf) << 16)
 #define CUBERT_SPLITS(n) (((n) & 0xff) << 8)
 #define CUBERT_SPLITS_OF(flags) (((flags) >> 8) & 0xff)
 size_t cubert_packed_bytes(size_t rows, size_t row_bytes);
