@@ -38,6 +38,14 @@ typedef struct Retval {
  * directory ("" -> model_npy/base_uncased or model_npy/large_uncased).
  * Precision and graph use come from the environment: CUBERT_PRECISION=fp32
  * (default) | bf16, CUBERT_GRAPH_MAX_TOKENS (default 8192, 0 disables graphs).
+ * fp32 mode agrees with the reference model to 1e-3 max-abs.  bf16 mode stores
+ * the Linear kernels and the GEMM operands in bfloat16 (fp32 accumulation,
+ * residual stream, statistics and softmax): against the float32 model on the
+ * same checkpoint it is within 3e-2 on both outputs when the checkpoint's
+ * Linear kernels are bfloat16-representable, and for the 12-layer model in
+ * any case; on a 24-layer checkpoint that is not, the [B,S,H] sequence output
+ * is within about 4e-2 (pooled output 2e-2), of which 0.026-0.035 is the
+ * storage rounding of the weights alone, whatever computes on them.
  * Returns NULL on failure (the reference exits the process); the reason is
  * available from cubert_last_error(). */
 void* init_model(bool large, int num_gpu, int max_batchsize, int max_seq_length, char* dir);
