@@ -455,12 +455,220 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
         }
 }
 
+
+// ---------------------------------------------------------------------------
+// Short batches (bf16, S <= 512, V as [B, heads, S, 64]): with one workgroup per (batch, head) a batch of one
+// occupies 16 CUs and every wave walks all key blocks one after the other.  Here a workgroup owns one block
+// of 32 queries of one (batch, head) and its NW waves share the KEYS: wave w takes the key blocks w, w + NW, ...
+// Nothing is staged for the workgroup: a wave requests its Q fragments, its K fragments (straight into the
+// MFMA operand layout), its V rows and its mask values in one go, drops the V rows into wave-private LDS (the
+// transposing read of the kernel above needs them there) and runs the same block arithmetic.  Each wave ends
+// with a partial (reference exponent, row sum, context) per query; the partials meet in LDS and every thread
+// finishes 32 / NW features of one query: ctx = sum_w 2^(ref_w - max ref) o_w / sum_w 2^(ref_w - max ref) sum_w.
+// No key block is skipped: a masked key's probability underflows to exactly zero, and a wave whose blocks are
+// all masked gets weight zero, so rows past a sequence's length (stale but finite in the compact-row pass) never
+// reach a result.  K / V of a head are fetched once per query block, which only a short batch can afford.
+template <int NW>
+__global__ __launch_bounds__(NW * 64, 4) void attention_split_kernel(
+    const unsigned char* __restrict__ q, const unsigned char* __restrict__ k,
+    const unsigned char* __restrict__ v, const float* __restrict__ maskadd,
+    unsigned char* __restrict__ ctx, int heads, int S, int Sp, float scale_log2e, int ctx_packed,
+    const int* __restrict__ cu, int first_only) {
+    constexpr int OSTRIDE = 68;                          // floats per query row of a partial context
+    constexpr int OBYTES = 32 * OSTRIDE * 4;             // two V blocks (8 KiB) first, the partial context later
+    constexpr int WBYTES = OBYTES + 256;                 // + the mask values of the two key blocks in flight
+    __shared__ __attribute__((aligned(16))) unsigned char sW[NW * WBYTES];
+    __shared__ float sRef[NW][32], sSum[NW][32];
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g = lane >> 5;
+    const int h = blockIdx.x, b = blockIdx.y, q0 = blockIdx.z * 32;
+    const int qlen = cu ? cu[b + 1] - cu[b] : S;
+    if (q0 >= qlen) return;                              // the whole workgroup: no barrier has been met
+    const int nblk = Sp >> 5;
+    const size_t bh = (size_t)b * heads + h;
+    const unsigned char* qb = q + bh * S * 128;
+    const unsigned char* kb = k + bh * S * 128;
+    unsigned char* myV = sW + wave * WBYTES;
+    unsigned char* myM = myV + OBYTES;
+    // V rows and mask values go from memory into this wave's LDS without passing through registers
+    const __amdgpu_buffer_rsrc_t vres = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(v + bh * S * 128), 0, S * 128, 0x00020000);
+    const __amdgpu_buffer_rsrc_t mres = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(maskadd + (size_t)b * Sp), 0, Sp * 4, 0x00020000);
+
+    uint4 qf[4];
+    {
+        int qrow = q0 + l32;
+        qrow = qrow < qlen ? qrow : qlen - 1;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+            qf[kk] = *reinterpret_cast<const uint4*>(qb + (size_t)qrow * 128 + (2 * kk + g) * 16);
+    }
+    f32x16_t o[2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.0f;
+    float run_max = -INFINITY, run_sum = 0.0f;
+    // where my 8-byte piece of a transposing read lies in a V block (see attention_lds_kernel)
+    int vpiece[2];
+    {
+        const int i16 = l32 & 15, prow = 4 * g + (i16 >> 2), psw = (prow >> 1) & 3;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+            vpiece[db] = prow * 128 + (((2 * db + (l32 >> 4)) ^ psw) << 5) + (i16 & 3) * 8;
+    }
+
+    for (int kb0 = wave; kb0 < nblk; kb0 += 2 * NW) {
+        const int nb = (kb0 + NW < nblk) ? 2 : 1;
+        uint4 kf[2][4];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (j < nb) {
+                const int k0 = (kb0 + j * NW) * 32;
+                int krow = k0 + l32;
+                krow = krow < S ? krow : S - 1;          // rows S .. Sp-1 do not exist; their mask term is -inf
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk)
+                    kf[j][kk] = *reinterpret_cast<const uint4*>(kb + (size_t)krow * 128 + (2 * kk + g) * 16);
+                // LDS slot s = 64 i + lane of the block holds the 16-byte chunk ch of row s >> 3, where the slot's place
+                // in the row is ch with its 32-byte block permuted by the row bits (the layout of the kernel above)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int sl = lane + 64 * i, row = sl >> 3, pos = sl & 7;
+                    const int ch = ((((pos >> 1) ^ ((row >> 1) & 3)) << 1) | (pos & 1));
+                    int vrow = k0 + row;
+                    vrow = vrow < S ? vrow : S - 1;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(vres, (lds_ptr_t)(myV + j * 4096 + i * 1024), 16, vrow * 128 + ch * 16, 0, 0, 0);
+                }
+            }
+        }
+        // mask term of key l32 of block kb0 (lanes 0 .. 31) and of block kb0 + NW (lanes 32 .. 63; beyond the row: zero)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(mres, (lds_ptr_t)myM, 4, ((kb0 + g * NW) * 32 + l32) * 4, 0, 0, 0);
+        // Everything requested above is one round trip; nothing below may read this wave's LDS before it is over (the
+        // transposing reads are not ordered behind the memory-to-LDS loads by the compiler).
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (j < nb) {
+                f32x16_t sc;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) sc[e] = 0.0f;
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk)
+                    sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf[j][kk]),
+                                                                 __builtin_bit_cast(bf16x8_t, qf[kk]), sc, 0, 0, 0);
+                float blk_max = -INFINITY;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const f32x4_t m4 = *reinterpret_cast<const f32x4_t*>(myM + j * 128 + (8 * jj + 4 * g) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float t = fmaf(sc[4 * jj + e], scale_log2e, m4[e] * 1.4426950408889634f);
+                        sc[4 * jj + e] = t;
+                        blk_max = fmaxf(blk_max, t);
+                    }
+                }
+                blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+                if (__ballot(blk_max > run_max + 20.0f) != 0ull) {
+                    const float new_max = fmaxf(run_max, blk_max);
+                    const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);
+                    run_sum *= alpha;
+                    run_max = new_max;
+#pragma unroll
+                    for (int db = 0; db < 2; ++db)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+                }
+                float blk_sum = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float pv = __builtin_amdgcn_exp2f(sc[e] - run_max);
+                    sc[e] = pv;
+                    blk_sum += pv;
+                }
+                blk_sum += __shfl_xor(blk_sum, 32);
+                run_sum += blk_sum;
+#pragma unroll
+                for (int f = 0; f < 2; ++f) {
+                    bf16x8_t pf;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pf[e] = (__bf16)sc[8 * f + e];
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+                        const unsigned char* piece = myV + j * 4096 + vpiece[db] + 16 * f * 128;
+                        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            reinterpret_cast<__attribute__((address_space(3))) s16x4_t*>((__attribute__((address_space(3))) unsigned char*)piece));
+                        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            reinterpret_cast<__attribute__((address_space(3))) s16x4_t*>((__attribute__((address_space(3))) unsigned char*)(piece + 8 * 128)));
+                        const s16x8_t vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vf), pf, o[db], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- the partials meet: wave w's context as [query][feature] over its V space ----
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    {
+        float* myO = reinterpret_cast<float*>(myV);
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4_t w4 = {o[db][4 * j], o[db][4 * j + 1], o[db][4 * j + 2], o[db][4 * j + 3]};
+                *reinterpret_cast<f32x4_t*>(myO + l32 * OSTRIDE + 32 * db + 8 * j + 4 * g) = w4;
+            }
+        if (g == 0) { sRef[wave][l32] = run_max; sSum[wave][l32] = run_sum; }
+    }
+    __syncthreads();
+    constexpr int FPT = 32 / NW;                 // features per thread: 8 (16 bytes of bf16) or 4
+    constexpr int GQ = 64 / FPT;                 // threads per query
+    const int qi = tid / GQ, fg = tid % GQ;
+    const int qrow = q0 + qi;
+    if (qrow >= qlen || (first_only && qrow != 0)) return;
+    const int nw = nblk < NW ? nblk : NW;        // waves that held a key block
+    float top = -INFINITY;
+    for (int w = 0; w < nw; ++w) top = fmaxf(top, sRef[w][qi]);
+    float den = 0.0f, acc[FPT];
+#pragma unroll
+    for (int e = 0; e < FPT; ++e) acc[e] = 0.0f;
+    for (int w = 0; w < nw; ++w) {
+        const float wgt = __builtin_amdgcn_exp2f(sRef[w][qi] - top);
+        den = fmaf(wgt, sSum[w][qi], den);
+        const float* src = reinterpret_cast<const float*>(sW + w * WBYTES) + qi * OSTRIDE + fg * FPT;
+#pragma unroll
+        for (int e = 0; e < FPT; e += 4) {
+            const f32x4_t x4 = *reinterpret_cast<const f32x4_t*>(src + e);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[e + c] = fmaf(wgt, x4[c], acc[e + c]);
+        }
+    }
+    const float inv = 1.0f / den;
+    const size_t hidden = (size_t)heads * 64;
+    const size_t row = first_only ? (size_t)b : (cu ? (size_t)cu[b] : (size_t)b * S) + qrow;
+    const int kbyte = (h * 64 + fg * FPT) * 2;
+    unsigned char* dst = ctx_packed ? ctx + packed_offset((int)row, kbyte, (int)hidden * 2 / 64) : ctx + row * hidden * 2 + kbyte;
+#pragma unroll
+    for (int e = 0; e < FPT; e += 4) {
+        const bf16x4_t w4 = {(__bf16)(acc[e] * inv), (__bf16)(acc[e + 1] * inv), (__bf16)(acc[e + 2] * inv), (__bf16)(acc[e + 3] * inv)};
+        *reinterpret_cast<bf16x4_t*>(dst + e * 2) = w4;
+    }
+}
+
 }  // namespace
 
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd, void* ctx,
                       bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt, hipStream_t stream,
-                      const int* cu, bool v_rowmajor, bool first_only) {
+                      const int* cu, bool v_rowmajor, bool first_only, int variant) {
     const int fo = first_only ? 1 : 0;
+    if (variant < kAttnAuto || variant > kAttnSplitKeys || (variant > kAttnPerHead && !(v_rowmajor && elt == kBF16 && S <= 512))) {
+        set_error("attention: the key-split variants need bf16 operands, S <= 512 and V as [B, heads, S, 64]");
+        return false;
+    }
     if (ctx_packed && elt != kBF16) { set_error("attention: only a bf16 context can be packed"); return false; }
     const int cp = ctx_packed ? 1 : 0;
     if (elt != kBF16 && elt != kF32) { set_error("attention: bad operand type"); return false; }
@@ -481,6 +689,15 @@ bool launch_attention(const void* q, const void* k, const void* vt, const float*
     const unsigned char* kc = static_cast<const unsigned char*>(k);
     const unsigned char* vc = static_cast<const unsigned char*>(vt);
     unsigned char* cc = static_cast<unsigned char*>(ctx);
+    if (elt == kBF16 && S <= 512 && v_rowmajor &&
+        (variant == kAttnSplitKeys || (variant == kAttnAuto && (long)B * heads * ((S + 31) / 32) <= kAttnSplitMaxWorkgroups))) {
+        const dim3 grid(heads, B, first_only ? 1 : (S + 31) / 32);
+        if (grid.z > 65535) { set_error("attention: grid too large"); return false; }
+        hipLaunchKernelGGL(attention_split_kernel<4>, grid, dim3(256), 0, stream, qc, kc, vc, maskadd, cc, heads, S, Sp,
+                           scale * 1.4426950408889634f, cp, cu, fo);
+        CUBERT_HIP_OK(hipGetLastError());
+        return true;
+    }
     if (elt == kBF16 && S <= 512) {
         const int vstride = round_up(Sp * 2, 256) + 8;
         const size_t lds = (size_t)Sp * 128 + (v_rowmajor ? (size_t)Sp * 128 : 64 * (size_t)vstride) + (size_t)Sp * 4 + 64;

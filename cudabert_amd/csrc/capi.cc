@@ -62,6 +62,7 @@ void* make_model(const cubert_config& cfg, int gpu, int maxB, int maxS, const ch
     opt.fuse_residual = env_int("CUBERT_FUSE_RESIDUAL", 1) != 0;
     opt.fuse_layernorm = env_int("CUBERT_FUSE_LAYERNORM", 1) != 0;
     opt.v_rowmajor = env_int("CUBERT_V_ROWMAJOR", 1) != 0;
+    opt.attn_split_workgroups = env_int("CUBERT_ATTN_SPLIT_WORKGROUPS", cubert::kAttnSplitMaxWorkgroups);
     opt.first_token_last_layer = env_int("CUBERT_FIRST_TOKEN_LAST_LAYER", 1) != 0;
     opt.gpu = gpu;
     opt.max_batch = maxB;
@@ -343,7 +344,8 @@ int cubert_op_attention(const void* q, const void* k, const void* vt, const floa
     cubert::set_error("");
     return cubert::launch_attention(q, k, vt, maskadd, ctx, (flags & CUBERT_Y_PACKED) != 0, B, heads, S,
                                     cubert::round_up(S > 0 ? S : 1, 32), scale, elt,
-                                    static_cast<hipStream_t>(stream), nullptr, (flags & CUBERT_V_ROWMAJOR) != 0) ? 0 : 1;
+                                    static_cast<hipStream_t>(stream), nullptr, (flags & CUBERT_V_ROWMAJOR) != 0, false,
+                                    (flags >> 20) & 3) ? 0 : 1;
 }
 
 int cubert_op_add_layernorm(float* x, const void* y, int y_elt, const float* gamma, const float* beta, void* xb,

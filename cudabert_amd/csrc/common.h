@@ -44,6 +44,10 @@ inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 // ds_read_b128 fragment reads (lane = row, 64-byte row pitch) run at the full
 // 256 bytes per clock of the LDS; measured alternatives: none 85, xor of
 // (r>>1)^(r>>3) 158 bytes per clock.
+// Attention kernels (launch_attention's `variant`).
+constexpr int kAttnAuto = 0, kAttnPerHead = 1, kAttnSplitKeys = 2;
+constexpr int kAttnSplitMaxWorkgroups = 768; // B * heads * ceil(S / 32) up to which kAttnAuto takes the key-split kernel
+
 __host__ __device__ inline int packed_swizzle(int r) { return (r >> 2) & 3; }
 __host__ __device__ inline size_t packed_bytes(size_t rows, size_t row_bytes) {
     return (rows + 255) / 256 * (row_bytes / 64) * 16384;

@@ -373,6 +373,7 @@ bool Model::run_compact(const int* lens, int B, int S) {
     const size_t cu_off = cap + 256 * (kMaxParts - 1);
     CUBERT_HIP_OK(hipMemcpyAsync(d_meta_ + cu_off, h_meta_ + cu_off, (size_t)parts * kCuStride * 4, hipMemcpyHostToDevice, stream_));
     cur_parts_ = parts;
+    cur_attn_ = (long)B * opt_.dims.heads * ((S + 31) / 32) <= opt_.attn_split_workgroups ? kAttnSplitKeys : kAttnPerHead;
     if (parts == 1) return enqueue_part(0, 0, B, 0, S, false, stream_, &cp[0]);
     CUBERT_HIP_OK(hipEventRecord(ev_fork_, stream_));
     bool ok = true;
@@ -482,6 +483,7 @@ void Model::forget_uncaptured_shapes() {
 // bandwidth-bound row kernel) another part's kernel takes the idle CUs.
 bool Model::enqueue(int B, int S, bool has_mask) {
     const long tokens = (long)B * S;
+    cur_attn_ = (long)B * opt_.dims.heads * ((S + 31) / 32) <= opt_.attn_split_workgroups ? kAttnSplitKeys : kAttnPerHead;
     int parts = opt_.split_parts < kMaxParts ? opt_.split_parts : kMaxParts;
     if (parts > B) parts = B;
     if (profiling_ || parts < 2 || opt_.split_min_tokens <= 0 || tokens < opt_.split_min_tokens) {
@@ -589,7 +591,7 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
             unsigned char* ctxc = static_cast<unsigned char*>(ctxc_) + c0 * H * es;
             unsigned char* hc = static_cast<unsigned char*>(hc_) + c0 * I * es;
             const void* xcin = elt == kBF16 ? static_cast<const void*>(xbc) : static_cast<const void*>(xc);
-            if (!launch_attention(q, k, vt, maskadd, ctxc, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow, true)) return false;
+            if (!launch_attention(q, k, vt, maskadd, ctxc, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow, true, vrow ? cur_attn_ : kAttnAuto)) return false;
             if (!launch_gather_first_rows(x32, cu, xc, B, S, H, st)) return false;
             g = GemmParams();
             g.elt = elt; g.out_elt = kF32; g.X = ctxc; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = yc;
@@ -612,7 +614,7 @@ bool Model::enqueue_part(int part, int b0, int B, size_t r0, int S, bool has_mas
             if (!mark(kPhPooler)) return false;
             return launch_pooler(xc, w_pool_, elt, b_pool_, pooled_ + (size_t)b0 * H, B, 1, H, st, nullptr);
         }
-        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow)) return false;
+        if (!launch_attention(q, k, vt, maskadd, ctx, pk, B, D.heads, S, Sp, scale, elt, st, cu, vrow, false, vrow ? cur_attn_ : kAttnAuto)) return false;
         // attention output projection -> f32, then residual add + LayerNorm
         g = GemmParams();
         g.elt = elt; g.out_elt = kF32; g.X = ctx; g.ldx = H; g.W = L.w_ao; g.bias = L.b_ao; g.Y = y32;

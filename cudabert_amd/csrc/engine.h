@@ -30,6 +30,9 @@ struct ModelOptions {
     bool fuse_residual = true;     // residual add in the epilogue of the GEMM before each LayerNorm
     bool fuse_layernorm = true;    // ... and the LayerNorm itself, where the GEMM kernel supports it (bf16, large batches)
     bool v_rowmajor = true;        // bf16, S <= 512: V is stored [B, heads, S, 64] like K; attention transposes on its LDS reads
+    int attn_split_workgroups = kAttnSplitMaxWorkgroups;   // bf16, S <= 512, row-major V: batches of up to this many
+                                   // (batch, head, 32 queries) blocks run the attention kernel that splits a head's keys
+                                   // over a workgroup's waves (0: never)
     bool split_k = true;           // short batches: split K of the hidden-wide GEMMs (changes the summation order)
     int varlen = -1;               // host-input calls with prefix masks compute only the valid tokens: 1 always,
                                    // 0 never, -1 when the caller asks for no sequence output (see forward_host)
@@ -148,6 +151,7 @@ class Model {
     bool first_only_ = false;                      // the pass being enqueued (and the last one run) is of that kind
     bool last_compact_ = false;
     int cur_parts_ = 1;          // parts of the pass being enqueued
+    int cur_attn_ = kAttnPerHead;   // attention kernel of the pass being enqueued (decided on the whole batch)
     int B_ = 0, S_ = 0;
     // hipGraph cache: one entry per (B, S, mask) shape, captured on second sight, at most
     // opt_.graph_cache instantiated at a time (least recently used goes first).

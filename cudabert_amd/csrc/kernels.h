@@ -113,8 +113,12 @@ bool gemm_ln_supported(int M, int N, int K, int elt);
 // ctx_packed (bf16 only): write ctx in the packed GEMM-operand layout (common.h).
 bool launch_attention(const void* q, const void* k, const void* vt, const float* maskadd,
                       void* ctx, bool ctx_packed, int B, int heads, int S, int Sp, float scale, int elt,
-                      hipStream_t stream, const int* cu = nullptr, bool v_rowmajor = false, bool first_only = false);
+                      hipStream_t stream, const int* cu = nullptr, bool v_rowmajor = false, bool first_only = false,
+                      int variant = kAttnAuto);
 // v_rowmajor (bf16, S <= 512 only): `vt` holds V as [B, heads, S, 64] like k.
+// variant (v_rowmajor only): kAttnPerHead = one workgroup per (batch, head); kAttnSplitKeys = one workgroup per
+// (batch, head, 32 queries) whose four waves share the keys: the short-batch kernel; kAttnAuto picks by the number of such workgroups.
+// The variants agree to the last bit or two of the bf16 context, not bit for bit.
 // first_only: only the context of every sequence's first token is produced, as row b of ctx [B, heads*64] (same bits
 // as row b * S of the full result).
 

@@ -194,6 +194,9 @@ long cubert_capacity_tokens(void* model);
 #define CUBERT_LN_NO_RESIDUAL 16    /* cubert_op_add_layernorm: y already contains the residual stream */
 #define CUBERT_V_ROWMAJOR 32        /* cubert_op_gemm_qkv / cubert_op_attention (bf16, S <= 512): the `vt` argument holds V as
                                        [B, heads, S, 64] like k instead of transposed */
+/* cubert_op_attention with CUBERT_V_ROWMAJOR: which kernel.  0 (no flag) = by batch size; 1 = one workgroup per
+ * (batch, head); 2 = one workgroup per (batch, head, 32 queries) whose four waves share the keys (short batches). */
+#define CUBERT_ATTN_VARIANT(n) (((n) & 3) << 20)
 /* Split K (cubert_op_gemm, epilogue 0, float32 Y): n workgroups share a tile, each reduces 1/n of K
  * and writes its partial sum to Y + i * M * N (the bias is in partial 0); Y holds n * M * N floats and
  * the consumer adds the parts (cubert_op_add_layernorm takes the count in the same flag bits). */

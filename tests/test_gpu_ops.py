@@ -12,6 +12,13 @@ F32, BF16 = 0, 1
 V_ROWMAJOR = 32          # CUBERT_V_ROWMAJOR
 
 
+def ATTN_VARIANT(n):      # CUBERT_ATTN_VARIANT: 1 = one workgroup per (batch, head), 2 = the waves of a workgroup share the keys
+    return (n & 3) << 20
+
+
+ATTN_SPLIT_MAX_WORKGROUPS = 768      # what cubert_op_attention decides by when no variant is named
+
+
 @pytest.fixture(scope="module")
 def pb():
     assert torch.cuda.is_available(), "GPU tests need a GPU"
@@ -182,8 +189,33 @@ def test_gemm_qkv_layouts(pb, elt, B, S, heads, tile, v_rowmajor):
     assert (vt_h[..., S:] == 0).all()                    # padding columns untouched
 
 
+def check_key_split_attention(pb, qd, kd, vr, md, per_head, ref, B, heads, S, scale, lens):
+    """The short-batch kernel (one workgroup per 32 queries of a head, its waves share the keys) against the float64
+    reference and against the one-workgroup-per-head kernel's result `per_head`: they sum in different orders, so they
+    agree to a bf16 rounding step or two, not bit for bit.  Without a named variant the entry point takes the
+    key-split kernel up to ATTN_SPLIT_MAX_WORKGROUPS blocks of 32 queries and the per-head one beyond."""
+    split = torch.full_like(per_head, float("nan"))
+    pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vr.data_ptr(), md.data_ptr(), split.data_ptr(),
+                                        B, heads, S, scale, BF16, V_ROWMAJOR | ATTN_VARIANT(2), stream()))
+    auto = torch.full_like(per_head, float("nan"))
+    pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vr.data_ptr(), md.data_ptr(), auto.data_ptr(),
+                                        B, heads, S, scale, BF16, V_ROWMAJOR, stream()))
+    torch.cuda.synchronize()
+    got = split.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    err = np.abs(got - ref).reshape(B, S, -1).max(axis=(1, 2))
+    for b in range(B):
+        assert err[b] < (5e-3 if lens is not None and lens[b] == 0 else 2e-2), (b, err[b])
+    diff = np.abs(got - per_head.float().cpu().numpy()).reshape(B, S, -1).max(axis=(1, 2))
+    for b in range(B):
+        if lens is None or lens[b] > 0:
+            assert diff[b] <= 2 * 2.0 ** -7, (b, diff[b])       # values of size 1..2 come in steps of 2^-7
+    taken = split if B * heads * ((S + 31) // 32) <= ATTN_SPLIT_MAX_WORKGROUPS else per_head
+    assert torch.equal(auto.view(torch.int16), taken.view(torch.int16))
+
+
 @pytest.mark.parametrize("elt", [F32, BF16])
-@pytest.mark.parametrize("B,S,heads", [(2, 5, 2), (3, 33, 2), (2, 200, 3), (1, 512, 2), (4, 128, 12)])
+@pytest.mark.parametrize("B,S,heads", [(2, 5, 2), (3, 33, 2), (2, 200, 3), (1, 512, 2), (4, 128, 12), (9, 200, 3), (12, 200, 12)])
 def test_attention(pb, elt, B, S, heads):
     print("attention", elt, B, S, heads, flush=True)
     rng = np.random.default_rng(S * 3 + B)
@@ -226,9 +258,10 @@ def test_attention(pb, elt, B, S, heads):
         vr = dev(v, tdt)
         ctx2 = torch.full((B * S, heads * 64), float("nan"), dtype=tdt, device="cuda")
         pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vr.data_ptr(), md.data_ptr(), ctx2.data_ptr(),
-                                            B, heads, S, scale, elt, V_ROWMAJOR, stream()))
+                                            B, heads, S, scale, elt, V_ROWMAJOR | ATTN_VARIANT(1), stream()))
         torch.cuda.synchronize()
         assert torch.equal(ctx.view(torch.int16), ctx2.view(torch.int16))
+        check_key_split_attention(pb, qd, kd, vr, md, ctx2, ref, B, heads, S, scale, lens)
     else:
         assert pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), md.data_ptr(), ctx.data_ptr(),
                                           B, heads, S, scale, elt, V_ROWMAJOR, stream()) != 0      # bf16 only
@@ -575,9 +608,10 @@ def test_attention_random_shapes(pb):
         vr = dev(v, torch.bfloat16)
         ctx2 = torch.full((B * S, heads * 64), float("nan"), dtype=torch.bfloat16, device="cuda")
         pb.check(pb.lib.cubert_op_attention(qd.data_ptr(), kd.data_ptr(), vr.data_ptr(), md.data_ptr(), ctx2.data_ptr(),
-                                            B, heads, S, 0.125, BF16, V_ROWMAJOR, stream()))
+                                            B, heads, S, 0.125, BF16, V_ROWMAJOR | ATTN_VARIANT(1), stream()))
         torch.cuda.synchronize()
         assert torch.equal(ctx.view(torch.int16), ctx2.view(torch.int16)), case
+        check_key_split_attention(pb, qd, kd, vr, md, ctx2, ref, B, heads, S, 0.125, None)
 
 
 LN_NO_RESIDUAL = 16
