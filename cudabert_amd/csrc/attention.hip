@@ -609,6 +609,8 @@ __global__ __launch_bounds__(NW * 64, 4) void attention_split_kernel(
                 }
             }
         }
+        // the next round's memory-to-LDS loads stay behind this round's LDS reads
+        asm volatile("" ::: "memory");
     }
 
     // ---- the partials meet: wave w's context as [query][feature] over its V space ----

@@ -292,6 +292,21 @@ __global__ __launch_bounds__(256) void mask_softmax_kernel(unsigned char* __rest
     }
 }
 
+// Maximum / sum over a group of `lpr` (8, 16, 32 or 64; wave-uniform) consecutive lanes, result in every lane of the
+// group: quad permutes, the mirrors of 8 and of 16 lanes, a swizzle for the other half of 32 and one exchange across
+// the halves of the wave -- no trip through the LDS crossbar until the last two.
+template <bool MAX>
+__device__ __forceinline__ float lane_group_reduce(float v, int lpr) {
+    auto comb = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+    v = comb(v, ln_dpp_lanes<0xB1>(v));        // lane ^ 1
+    v = comb(v, ln_dpp_lanes<0x4E>(v));        // lane ^ 2
+    v = comb(v, ln_dpp_lanes<0x141>(v));       // the other quad of 8 lanes
+    if (lpr >= 16) v = comb(v, ln_dpp_lanes<0x140>(v));       // the other 8 of 16 lanes
+    if (lpr >= 32) v = comb(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));   // lane ^ 16
+    if (lpr >= 64) v = comb(v, __shfl_xor(v, 32));
+    return v;
+}
+
 // Vectorised form for rows whose byte length is a multiple of 16 (S % 4 == 0 for
 // float32, S % 8 == 0 for bf16): a row is cut into 16-byte chunks, a group of LPR
 // lanes (a power of two, 8..64) owns one row and each lane U chunks, so a wave
@@ -371,7 +386,7 @@ __global__ __launch_bounds__(256) void mask_softmax_vec_kernel(unsigned char* __
                 for (int e = 0; e < EPC; ++e) v[u][e] = -INFINITY;
             }
         }
-        for (int m = lpr >> 1; m > 0; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
+        mx = lane_group_reduce<true>(mx, lpr);
         if (!live) mx = 0.0f;                      // keeps exp(-inf - mx) well defined for absent rows
         float sum = 0.0f;
 #pragma unroll
@@ -381,7 +396,7 @@ __global__ __launch_bounds__(256) void mask_softmax_vec_kernel(unsigned char* __
                 v[u][e] = __builtin_amdgcn_exp2f(v[u][e] - mx);     // 0 for the chunks this lane does not own
                 sum += v[u][e];
             }
-        for (int m = lpr >> 1; m > 0; m >>= 1) sum += __shfl_xor(sum, m);
+        sum = lane_group_reduce<false>(sum, lpr);
         const float inv = 1.0f / sum;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
