@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void attention_kernel(
                 blk_max = fmaxf(blk_max, s);
             }
         }
-        blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+        blk_max = half_swap_max(blk_max);
         const float new_max = fmaxf(run_max, blk_max);    // finite: key 0 is never padding
         const float alpha = __expf(run_max - new_max);    // exp(-inf) = 0 on the first block
         float blk_sum = 0.0f;
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void attention_kernel(
             sc[v] = pv;
             blk_sum += pv;
         }
-        blk_sum += __shfl_xor(blk_sum, 32);
+        blk_sum = half_swap_sum(blk_sum);
         run_sum = run_sum * alpha + blk_sum;
         run_max = new_max;
 #pragma unroll
@@ -376,7 +376,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
                 }
             }
         }
-        blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+        blk_max = half_swap_max(blk_max);
         if (__ballot(blk_max > run_max + 20.0f) != 0ull) {    // finite blk_max: a processed block holds a real key column
             const float new_max = fmaxf(run_max, blk_max);
             const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);     // 1 for the lanes that stay
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(1024) void attention_lds_kernel(
                 blk_sum += pv;
             }
         }
-        blk_sum += __shfl_xor(blk_sum, 32);
+        blk_sum = half_swap_sum(blk_sum);
         run_sum += blk_sum;
 
         // ---- ctx^T += V^T (rows = head features) x P^T (column = my query) ----
@@ -571,7 +571,7 @@ __global__ __launch_bounds__(NW * 64, 4) void attention_split_kernel(
                         blk_max = fmaxf(blk_max, t);
                     }
                 }
-                blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+                blk_max = half_swap_max(blk_max);
                 if (__ballot(blk_max > run_max + 20.0f) != 0ull) {
                     const float new_max = fmaxf(run_max, blk_max);
                     const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);
@@ -589,7 +589,7 @@ __global__ __launch_bounds__(NW * 64, 4) void attention_split_kernel(
                     sc[e] = pv;
                     blk_sum += pv;
                 }
-                blk_sum += __shfl_xor(blk_sum, 32);
+                blk_sum = half_swap_sum(blk_sum);
                 run_sum += blk_sum;
 #pragma unroll
                 for (int f = 0; f < 2; ++f) {

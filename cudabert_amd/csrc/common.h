@@ -79,6 +79,25 @@ __device__ __forceinline__ float ln_dpp_lanes(float v) {
 }
 // Sum over the 32 lanes that share lane / 32; every lane gets the same bits (the additions are
 // pairwise and commutative).
+// v combined with the value of the lane 32 further (or back): gfx950's v_permlane32_swap exchanges the upper half of
+// one register with the lower half of another, so of two copies of v one ends up holding v of the lower lane of each
+// pair in both halves and the other v of the upper lane; sum and maximum commute, so the result has the bits of
+// v + shfl_xor(v, 32) / max(v, shfl_xor(v, 32)) without the trip through the LDS crossbar.  (Inline asm, with the wait
+// states the instruction needs after a vector write of its operands and before a vector read of its results: the
+// compiler's builtin returns the first register twice.)
+__device__ __forceinline__ void half_swap(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float half_swap_sum(float v) {
+    float a = v, b = v;
+    half_swap(a, b);
+    return a + b;
+}
+__device__ __forceinline__ float half_swap_max(float v) {
+    float a = v, b = v;
+    half_swap(a, b);
+    return fmaxf(a, b);
+}
 __device__ __forceinline__ float ln_half_wave_sum(float v) {
     v += ln_dpp_lanes<0xB1>(v);       // quad_perm [1,0,3,2]: lane ^ 1
     v += ln_dpp_lanes<0x4E>(v);       // quad_perm [2,3,0,1]: lane ^ 2

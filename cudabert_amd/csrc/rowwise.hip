@@ -14,13 +14,15 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 constexpr int kMaxChunks = 4;        // 4 chunks x 64 lanes x 4 elements = rows up to 1024
 
 __device__ __forceinline__ float wave_sum(float v) {
+    v = half_swap_sum(v);
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o);
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
+    v = half_swap_max(v);
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
     return v;
 }
 
@@ -303,7 +305,7 @@ __device__ __forceinline__ float lane_group_reduce(float v, int lpr) {
     v = comb(v, ln_dpp_lanes<0x141>(v));       // the other quad of 8 lanes
     if (lpr >= 16) v = comb(v, ln_dpp_lanes<0x140>(v));       // the other 8 of 16 lanes
     if (lpr >= 32) v = comb(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));   // lane ^ 16
-    if (lpr >= 64) v = comb(v, __shfl_xor(v, 32));
+    if (lpr >= 64) v = MAX ? half_swap_max(v) : half_swap_sum(v);
     return v;
 }
 
