@@ -183,6 +183,34 @@ def test_base_cfg0_bf16(pb, base_dir):
 
 
 @pytest.mark.parametrize("precision", [F32, BF16])
+def test_largest_batch_the_reference_allows(pb, tiny_dir, precision):
+    """B = 1024 is the reference's ceiling (cuda_bert/ops/batch_matmul.cu:60; manager.cu:100-108): it runs, with the
+    ragged lengths of a real batch, padded and (host entry, pooled output only) on the valid tokens; one sequence
+    more is refused with an error, not a crash."""
+    wdir = str(tiny_dir / ("f32" if precision == F32 else "bf16"))
+    npy = W.load_npy_dir(wdir)
+    B, S = 1024, 12
+    rng = np.random.default_rng(3)
+    lens = rng.integers(1, S + 1, size=B)
+    lens[0] = S
+    ids, seg, mask = synth.make_inputs(B, S, list(lens), vocab=W.TINY.vocab, seed=9, prune=False)
+    seq_ref, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+    m = load(pb, W.TINY, wdir, precision, 1025, S)
+    try:
+        pooled, seq, _ = pb.encode(m, ids, seg, mask, want_seq=True)
+        pooled_only, _, _ = pb.encode(m, ids, seg, mask)
+        more = np.zeros((1025, S), np.int32)
+        with pytest.raises(pb.CubertError, match="1024"):
+            pb.encode(m, more, more, more)
+    finally:
+        pb.unload_model(m)
+    valid = mask.astype(bool)
+    assert np.abs(seq - seq_ref)[valid].max() < TOL[precision]
+    assert np.abs(pooled - pooled_ref).max() < TOL[precision]
+    assert np.abs(pooled_only - pooled_ref).max() < TOL[precision]
+
+
+@pytest.mark.parametrize("precision", [F32, BF16])
 def test_base_max_position_length(pb, base_dir, precision):
     """Sequences at the position table's limit (S = 512) with the skewed lengths of benchmark
     configuration 4: one long, the others short; also B = 1."""
