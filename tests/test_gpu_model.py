@@ -112,6 +112,34 @@ def test_reference_entry_points(pb, tiny_dir):
         pb.unload_model(m)
 
 
+def test_empty_and_malformed_calls_are_errors(pb, tiny_dir):
+    """Nothing to compute, nothing to read from, or nothing to write to: an error code and a message, the model stays
+    usable.  (The reference asserts on shapes, cuda_bert/utils/manager.cu:100-108, and dereferences the rest.)"""
+    wdir = str(tiny_dir / "f32")
+    npy = W.load_npy_dir(wdir)
+    m = load(pb, W.TINY, wdir, F32, 4, 32)
+    try:
+        ids, seg, mask = synth.make_inputs(2, 16, [16, 5], vocab=W.TINY.vocab, seed=2, prune=False)
+        out = np.empty((2, W.TINY.hidden), np.float32)
+        enc = pb.lib.cubert_encode
+        p = lambda a: a.ctypes.data
+        assert enc(m, p(ids), p(seg), p(mask), 0, 16, p(out), None, None) != 0 and b"positive" in pb.lib.cubert_last_error()
+        assert enc(m, p(ids), p(seg), p(mask), 2, 0, p(out), None, None) != 0 and b"positive" in pb.lib.cubert_last_error()
+        assert enc(m, p(ids), p(seg), p(mask), -1, 16, p(out), None, None) != 0
+        assert enc(m, None, p(seg), p(mask), 2, 16, p(out), None, None) != 0 and b"null" in pb.lib.cubert_last_error()
+        assert enc(m, p(ids), None, p(mask), 2, 16, p(out), None, None) != 0
+        assert enc(None, p(ids), p(seg), p(mask), 2, 16, p(out), None, None) != 0
+        neg = seg.copy()
+        neg[0, 0] = -1
+        assert enc(m, p(ids), p(neg), p(mask), 2, 16, p(out), None, None) != 0 and b"token type" in pb.lib.cubert_last_error()
+        # and after all that a good call still gives the right answer
+        pooled, _, _ = pb.encode(m, ids, seg, mask)
+        _, pooled_ref = O.forward_torch(npy, W.TINY.heads, ids, seg, mask)
+        assert np.abs(pooled - pooled_ref).max() < TOL[F32]
+    finally:
+        pb.unload_model(m)
+
+
 def test_device_inputs_and_graph_replay(pb, tiny_dir):
     wdir = str(tiny_dir / "f32")
     npy = W.load_npy_dir(wdir)
